@@ -7,6 +7,8 @@ hand-written HIP kernels under ``csrc/``.
 """
 from . import registry
 from .parts import standard as _standard_parts   # registers the parts
+from .parts import hybrid as _hybrid_parts       # registers the parallel block, the mixers with a memory, routed experts
 from .architectures import llama as _llama       # registers LlamaForCausalLM
+from .architectures import zekalorn as _zekalorn  # registers Zekalorn
 
 __version__ = "0.1.0"

@@ -167,9 +167,10 @@ class KVCacheManager:
         if device is not None:
             for g in self.groups:
                 shape = (g.pages.num_pages, g.need.kv_heads, self.page_size, g.need.head_dim)
+                vshape = shape[:3] + (g.need.value_dim,)
                 for cid in g.cache_ids:
                     g.kpools[cid] = torch.zeros(shape, dtype=dtype, device=device)
-                    g.vpools[cid] = torch.zeros(shape, dtype=dtype, device=device)
+                    g.vpools[cid] = torch.zeros(vshape, dtype=dtype, device=device)
             for cid, sn in self.state_needs.items():
                 self.state[cid] = torch.zeros((max_requests,) + tuple(sn.shape), dtype=sn.dtype, device=device)
 
@@ -209,15 +210,16 @@ class KVCacheManager:
     def pool_bytes(self) -> int:
         """Bytes of all key and value pools together."""
         el = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(2 * len(g.cache_ids) * g.pages.num_pages * g.need.kv_heads * self.page_size * g.need.head_dim * el
-                   for g in self.groups)
+        return sum(len(g.cache_ids) * g.pages.num_pages * g.need.kv_heads * self.page_size
+                   * (g.need.head_dim + g.need.value_dim) * el for g in self.groups)
 
     @staticmethod
     def pages_for_bytes(needs: Dict[int, CacheNeed], page_size: int, budget_bytes: int, dtype: torch.dtype) -> int:
         """The largest ``num_pages`` whose pools fit ``budget_bytes`` when every cache of ``needs`` that
         holds keys and values gets that many pages (windowed groups may then be given fewer)."""
         el = torch.empty(0, dtype=dtype).element_size()
-        per_page = sum(2 * n.kv.kv_heads * page_size * n.kv.head_dim * el for n in needs.values() if n.kv is not None)
+        per_page = sum(n.kv.kv_heads * page_size * (n.kv.head_dim + n.kv.value_dim) * el
+                       for n in needs.values() if n.kv is not None)
         return int(budget_bytes // per_page) if per_page else 0
 
     def utilization(self) -> float:

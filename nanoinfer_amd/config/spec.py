@@ -57,6 +57,9 @@ class LayerRun:
     block: int
     cache: int
     writes_cache: bool = True
+    # row of the model's ``pass_input`` (a part of family ``pass_input``) that is added to the residual
+    # stream right before this entry runs: the mark of a new pass over a run of blocks that is repeated
+    enter: Optional[int] = None
 
 
 @dataclass
@@ -77,6 +80,8 @@ class ModelSpec:
     # endings of tensor names that a checkpoint may hold without the model asking for them (buffers that
     # exporters write along, such as a rotation's stored frequencies); they are not loaded
     ignorable_suffixes: tuple = ()
+    # what entries of the order with ``enter`` add to the stream (None: no entry has one)
+    pass_input: Optional[PartSpec] = None
 
     def num_caches(self) -> int:
         return 1 + max((r.cache for r in self.order), default=-1)

@@ -1,0 +1,224 @@
+// Causal softmax attention over the paged cache with a bias by distance and a query temperature,
+// keys and values of different sizes, for gfx950.
+//
+//     score(i, j) = (q_i . k_j) * scale * temp(i) + bias[i - j, head]      for j <= i
+//     temp(p) = 1 + coef * ln(floor((p + 1) / every) + 1)
+//
+// `bias` is a float32 table [distances, heads] that the host has laid out from the learned rows (one
+// row for every distance up to the model's last position), so the kernel needs no logarithm a score.
+// Pools are [page, kv_head, slot_in_page, size] with size dk for keys and dv for values.
+//
+// One workgroup of four wavefronts takes a tile of consecutive tokens of one sequence and (a chunk of)
+// the query heads of one kv head: 16 rows of (token, head), four a wavefront.  64 keys and values at a
+// time are staged in LDS as float32 for the whole workgroup; a lane owns one key of the 64 for the
+// scores of its wavefront's four rows, then one value channel (and the ones 64 further on) for the
+// weighted sum.  Everything is float32; the softmax is the running one (maximum, sum, rescaled sum).
+#include "common.h"
+
+#include <algorithm>
+#include <cmath>
+
+#define ROWS_PER_WAVE 4
+#define WAVES 4
+#define ROWS (ROWS_PER_WAVE * WAVES)
+#define KEYS 64
+#define MAX_VCHUNKS 4          // value channels a lane owns at most: dv <= 256
+
+// keys and values of the step's tokens into their places in the pages
+template <typename T>
+__global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k_off, int v_off,
+                                const int32_t* __restrict__ slot_mapping, T* __restrict__ kpool, T* __restrict__ vpool,
+                                int G, int dk, int dv, int page_size) {
+    const int t = blockIdx.x;
+    const int slot = slot_mapping[t];
+    if (slot < 0) return;
+    const int page = slot / page_size, in_page = slot % page_size;
+    const T* row = qkv + static_cast<size_t>(t) * row_stride;
+    for (int i = threadIdx.x; i < G * dk; i += blockDim.x) {
+        const int g = i / dk, c = i % dk;
+        kpool[((static_cast<size_t>(page) * G + g) * page_size + in_page) * dk + c] = row[k_off + i];
+    }
+    for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
+        const int g = i / dv, c = i % dv;
+        vpool[((static_cast<size_t>(page) * G + g) * page_size + in_page) * dv + c] = row[v_off + i];
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(WAVES * WAVE)
+bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
+                      const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
+                      const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
+                      int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk) {
+    extern __shared__ float lds[];
+    const int dkp = dk + 1;                       // a lane reads its key's row: odd strides spread the banks
+    float* Qs = lds;                              // [ROWS][dk]
+    float* Ks = Qs + ROWS * dk;                   // [KEYS][dkp]
+    float* Vs = Ks + KEYS * dkp;                  // [KEYS][dv]
+    float* Ps = Vs + KEYS * dv;                   // [WAVES][ROWS_PER_WAVE][KEYS]
+    const int tile = blockIdx.x, g = blockIdx.y, chunk = blockIdx.z;
+    const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2], first_pos = tiles[4 * tile + 3];
+    const int group = H / G;
+    const int heads_here = std::min(heads_per_chunk, group - chunk * heads_per_chunk);
+    const int head0 = g * group + chunk * heads_per_chunk;
+    const int n_rows = n_tok * heads_here;        // row r = token r / heads_here, head r % heads_here
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+
+    for (int i = tid; i < ROWS * dk; i += blockDim.x) {
+        const int r = i / dk, c = i % dk;
+        float v = 0.f;
+        if (r < n_rows)
+            v = ld(qkv + static_cast<size_t>(first_row + r / heads_here) * row_stride + (head0 + r % heads_here) * dk + c);
+        Qs[i] = v;
+    }
+    float m[ROWS_PER_WAVE], l[ROWS_PER_WAVE], acc[ROWS_PER_WAVE][MAX_VCHUNKS], factor[ROWS_PER_WAVE];
+    int pos[ROWS_PER_WAVE], head[ROWS_PER_WAVE];
+    bool valid[ROWS_PER_WAVE];
+#pragma unroll
+    for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
+        const int r = wave * ROWS_PER_WAVE + rr;
+        valid[rr] = r < n_rows;
+        pos[rr] = first_pos + (valid[rr] ? r / heads_here : 0);
+        head[rr] = head0 + (valid[rr] ? r % heads_here : 0);
+        const int steps = temp_every > 0 ? (pos[rr] + 1) / temp_every : 0;
+        factor[rr] = scale * (1.0f + temp_coef * logf(static_cast<float>(steps) + 1.0f));
+        m[rr] = -INFINITY;
+        l[rr] = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < MAX_VCHUNKS; ++cc) acc[rr][cc] = 0.f;
+    }
+    const int last_pos = first_pos + n_tok - 1;
+    const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
+    for (int k0 = 0; k0 <= last_pos; k0 += KEYS) {
+        __syncthreads();                          // the tile before this one has been used by everyone
+        for (int i = tid; i < KEYS * dk; i += blockDim.x) {
+            const int j = i / dk, c = i % dk, key = k0 + j;
+            float v = 0.f;
+            if (key <= last_pos) {
+                const int page = table[key / page_size];
+                if (page >= 0) v = ld(kpool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * dk + c);
+            }
+            Ks[j * dkp + c] = v;
+        }
+        for (int i = tid; i < KEYS * dv; i += blockDim.x) {
+            const int j = i / dv, c = i % dv, key = k0 + j;
+            float v = 0.f;
+            if (key <= last_pos) {
+                const int page = table[key / page_size];
+                if (page >= 0) v = ld(vpool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * dv + c);
+            }
+            Vs[i] = v;
+        }
+        __syncthreads();
+        // scores of this lane's key for the wavefront's rows
+        float s[ROWS_PER_WAVE];
+#pragma unroll
+        for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) s[rr] = 0.f;
+        const float* krow = Ks + lane * dkp;
+        const float* qrow = Qs + wave * ROWS_PER_WAVE * dk;
+        for (int c = 0; c < dk; ++c) {
+            const float kv = krow[c];
+#pragma unroll
+            for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) s[rr] += qrow[rr * dk + c] * kv;
+        }
+        const int key = k0 + lane;
+        float* prow = Ps + wave * ROWS_PER_WAVE * KEYS;
+        float alpha[ROWS_PER_WAVE];
+#pragma unroll
+        for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
+            alpha[rr] = 1.f;
+            if (!valid[rr]) { prow[rr * KEYS + lane] = 0.f; continue; }          // the same for the whole wavefront
+            if (k0 > pos[rr]) { prow[rr * KEYS + lane] = 0.f; continue; }        // the same for the whole wavefront
+            const bool seen = key <= pos[rr];
+            float sc = -INFINITY;
+            if (seen) {
+                const int back = std::min(pos[rr] - key, distances - 1);
+                sc = s[rr] * factor[rr] + (bias ? bias[static_cast<size_t>(back) * H + head[rr]] : 0.f);
+            }
+            const float m_new = fmaxf(m[rr], wave_max(sc));      // finite: key k0 <= pos is seen
+            alpha[rr] = expf(m[rr] - m_new);                      // 0 at the first tile
+            const float p = seen ? expf(sc - m_new) : 0.f;
+            l[rr] = l[rr] * alpha[rr] + wave_sum(p);
+            m[rr] = m_new;
+            prow[rr * KEYS + lane] = p;
+        }
+        // a wavefront reads only what it wrote itself: no barrier of the workgroup is needed here
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int cc = 0; cc < MAX_VCHUNKS; ++cc) {
+            const int c = lane + cc * WAVE;
+            if (c < dv) {
+                float add[ROWS_PER_WAVE];
+#pragma unroll
+                for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) add[rr] = 0.f;
+                for (int j = 0; j < KEYS; ++j) {
+                    const float vv = Vs[j * dv + c];
+#pragma unroll
+                    for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) add[rr] += prow[rr * KEYS + j] * vv;
+                }
+#pragma unroll
+                for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) acc[rr][cc] = acc[rr][cc] * alpha[rr] + add[rr];
+            }
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
+        if (!valid[rr]) continue;
+        const int r = wave * ROWS_PER_WAVE + rr;
+        T* orow = out + static_cast<size_t>(first_row + r / heads_here) * (H * dv) + head[rr] * dv;
+        const float inv = 1.0f / l[rr];
+#pragma unroll
+        for (int cc = 0; cc < MAX_VCHUNKS; ++cc) {
+            const int c = lane + cc * WAVE;
+            if (c < dv) st(orow + c, acc[rr][cc] * inv);
+        }
+    }
+}
+
+NI_EXPORT int ni_kv_store(const void* qkv, int row_stride, int k_off, int v_off, const void* slot_mapping, void* kpool,
+                          void* vpool, int T, int G, int dk, int dv, int page_size, int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (dtype == 0)
+        kv_store_kernel<float><<<T, 256, 0, stream>>>((const float*)qkv, row_stride, k_off, v_off, (const int32_t*)slot_mapping,
+                                                      (float*)kpool, (float*)vpool, G, dk, dv, page_size);
+    else
+        kv_store_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)qkv, row_stride, k_off, v_off, (const int32_t*)slot_mapping,
+                                                       (bf16_t*)kpool, (bf16_t*)vpool, G, dk, dv, page_size);
+    return NI_LAUNCH_RESULT();
+}
+
+NI_EXPORT int ni_bias_attention_rows() { return ROWS; }
+
+NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
+                                int table_width, const void* tiles, int n_tiles, const void* bias, int distances, void* out,
+                                int H, int G, int dk, int dv, int page_size, float scale, float temp_coef, int temp_every,
+                                int heads_per_chunk, int dtype, hipStream_t stream) {
+    if (n_tiles <= 0) return 0;
+    if (dv > MAX_VCHUNKS * WAVE || H % G || heads_per_chunk < 1 || heads_per_chunk > ROWS) return -1;
+    const int group = H / G;
+    const size_t lds = (static_cast<size_t>(ROWS) * dk + static_cast<size_t>(KEYS) * (dk + 1) + static_cast<size_t>(KEYS) * dv +
+                        WAVES * ROWS_PER_WAVE * KEYS) * sizeof(float);
+    if (lds > 160 * 1024) return -2;
+    dim3 grid(n_tiles, G, (group + heads_per_chunk - 1) / heads_per_chunk);
+    hipError_t err = hipSuccess;
+    if (dtype == 0) {
+        static size_t allowed = 48 * 1024;
+        if (lds > allowed && (allowed = lds))
+            err = hipFuncSetAttribute((const void*)bias_attention_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return (int)err;
+        bias_attention_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
+            (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
+            (const int32_t*)tiles, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
+            temp_every, heads_per_chunk);
+    } else {
+        static size_t allowed = 48 * 1024;
+        if (lds > allowed && (allowed = lds))
+            err = hipFuncSetAttribute((const void*)bias_attention_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return (int)err;
+        bias_attention_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
+            (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
+            (const int32_t*)tiles, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
+            temp_every, heads_per_chunk);
+    }
+    return NI_LAUNCH_RESULT();
+}

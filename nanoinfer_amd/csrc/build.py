@@ -123,7 +123,26 @@ def library_path(name: str, sources: List[str], defines: Optional[Dict[str, obje
 CORE = ("ni_ops", ["ops.hip"], {})
 SAMPLING = ("ni_sampling", ["sampling.hip"], {})
 SKINNY = ("ni_skinny_gemm", ["gemv.hip"], {})
+STREAM_OPS = ("ni_stream_ops", ["stream_ops.hip"], {})
+BIAS_ATTENTION = ("ni_bias_attention", ["bias_attention.hip"], {})
 COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
+COMMON_DELTA_KEY_SIZES = (16, 32, 48, 64, 96, 128)
+
+
+def delta_rule_split(key_size: int):
+    """How the delta-rule kernel holds a column of its state: ``parts`` neighbouring lanes with
+    ``per_lane`` key channels each (parts a power of two, at most 16; parts * per_lane = key_size)."""
+    if not 1 <= key_size <= 256:
+        raise BuildError(f"key size {key_size} is not supported by the delta-rule kernel: 1 to 256")
+    parts = 16
+    while key_size % parts:
+        parts //= 2
+    return key_size // parts, parts
+
+
+def delta_rule_target(key_size: int):
+    per_lane, parts = delta_rule_split(key_size)
+    return (f"ni_delta_rule_k{key_size}", ["delta_rule.hip"], {"KPT": per_lane, "PARTS": parts})
 
 
 def attention_target(head_dim: int):
@@ -148,9 +167,10 @@ def attention_mfma_f32_target(head_dim: int):
 
 
 def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, verbose: bool = True,
-              jobs: Optional[int] = None) -> List[str]:
-    """Compile every library (attention for the given head sizes)."""
-    targets = [CORE, SAMPLING, SKINNY] + [attention_target(h) for h in head_dims] + \
+              jobs: Optional[int] = None, delta_key_sizes: Iterable[int] = COMMON_DELTA_KEY_SIZES) -> List[str]:
+    """Compile every library (attention for the given head sizes, the delta rule for the given key sizes)."""
+    targets = [CORE, SAMPLING, SKINNY, STREAM_OPS, BIAS_ATTENTION] + [delta_rule_target(k) for k in delta_key_sizes] + \
+        [attention_target(h) for h in head_dims] + \
         [attention_mfma_target(h) for h in head_dims] + \
         [attention_mfma_f32_target(h) for h in head_dims]
     # the compiler runs in processes of its own: a few at a time (the longest, the skinny product, first)

@@ -1,0 +1,290 @@
+// Kernels around the residual stream and the routed feed-forward for gfx950: an embedding that
+// scales its rows and adds a learned position row, sums onto the float32 stream, a token's side
+// input, the router's choice, and the products of the chosen experts for steps of few rows.
+//
+// Conventions as in ops.hip: the stream is float32, what feeds a matrix product is the compute
+// type (float or bfloat16), all arithmetic is float32, every entry point returns 0 or a hipError_t.
+#include "common.h"
+
+#include <algorithm>
+
+static inline unsigned blocks_of(size_t n, unsigned per) { return static_cast<unsigned>((n + per - 1) / per); }
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+    const float c = 0.7978845608028654f;
+    return 0.5f * z * (1.0f + tanhf(c * (z + 0.044715f * z * z * z)));
+}
+
+// ---------------------------------------------------------------- embedding: row * scale + position row
+template <typename T>
+__global__ void embed_scaled_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ positions,
+                                    const T* __restrict__ table, const T* __restrict__ pos_table, float* __restrict__ out,
+                                    int d, int vocab, int max_pos, float scale) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    if (id < 0 || id >= vocab) return;      // unreachable after the host's check
+    const T* row = table + static_cast<size_t>(id) * d;
+    float* o = out + static_cast<size_t>(t) * d;
+    const T* prow = nullptr;
+    if (pos_table) {
+        const int p = positions[t];
+        if (p < 0 || p >= max_pos) return;  // the runner refuses a request before it reaches the last position
+        prow = pos_table + static_cast<size_t>(p) * d;
+    }
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = ld(row + i) * scale;
+        if (prow) v += ld(prow + i);
+        o[i] = v;
+    }
+}
+
+NI_EXPORT int ni_embed_scaled(const void* ids, const void* positions, const void* table, const void* pos_table, void* out,
+                              int T, int d, int vocab, int max_pos, float scale, int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (dtype == 0)
+        embed_scaled_kernel<float><<<T, 256, 0, stream>>>((const int32_t*)ids, (const int32_t*)positions, (const float*)table,
+                                                          (const float*)pos_table, (float*)out, d, vocab, max_pos, scale);
+    else
+        embed_scaled_kernel<bf16_t><<<T, 256, 0, stream>>>((const int32_t*)ids, (const int32_t*)positions, (const bf16_t*)table,
+                                                           (const bf16_t*)pos_table, (float*)out, d, vocab, max_pos, scale);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- h[t, :] += vec
+__global__ void add_vector_kernel(float* __restrict__ h, const float* __restrict__ vec, int d, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) h[i] += vec[i % d];
+}
+
+NI_EXPORT int ni_add_vector(void* h, const void* vec, int T, int d, hipStream_t stream) {
+    const size_t n = static_cast<size_t>(T) * d;
+    if (n == 0) return 0;
+    add_vector_kernel<<<blocks_of(n, 256), 256, 0, stream>>>((float*)h, (const float*)vec, d, n);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- h += (a + b); x = h in the compute type
+// a and b (b may be absent) are float32 or the compute type; the two are added first, then the stream.
+template <typename TA, typename TB, typename TX>
+__global__ void stream_add_kernel(float* __restrict__ h, const TA* __restrict__ a, const TB* __restrict__ b,
+                                  TX* __restrict__ x, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = ld(a + i);
+    if (b) s += ld(b + i);
+    const float v = h[i] + s;
+    h[i] = v;
+    if (x) st(x + i, v);
+}
+
+template <typename TA, typename TB>
+static void launch_stream_add(float* h, const TA* a, const TB* b, void* x, int x_dtype, size_t n, hipStream_t stream) {
+    const unsigned blocks = blocks_of(n, 256);
+    if (x_dtype == 0)
+        stream_add_kernel<TA, TB, float><<<blocks, 256, 0, stream>>>(h, a, b, (float*)x, n);
+    else
+        stream_add_kernel<TA, TB, bf16_t><<<blocks, 256, 0, stream>>>(h, a, b, (bf16_t*)x, n);
+}
+
+NI_EXPORT int ni_stream_add(void* h, const void* a, int a_dtype, const void* b, int b_dtype, void* x, int x_dtype,
+                            int T, int d, hipStream_t stream) {
+    const size_t n = static_cast<size_t>(T) * d;
+    if (n == 0) return 0;
+    if (a_dtype == 0 && b_dtype == 0) launch_stream_add((float*)h, (const float*)a, (const float*)b, x, x_dtype, n, stream);
+    else if (a_dtype == 0) launch_stream_add((float*)h, (const float*)a, (const bf16_t*)b, x, x_dtype, n, stream);
+    else if (b_dtype == 0) launch_stream_add((float*)h, (const bf16_t*)a, (const float*)b, x, x_dtype, n, stream);
+    else launch_stream_add((float*)h, (const bf16_t*)a, (const bf16_t*)b, x, x_dtype, n, stream);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- g = gelu_tanh(z) * side_row
+// z float32 [T, width] (columns beyond `ds` are padding and give zeros); the side row of token t is
+// table[ids[t], first : first + ds].
+template <typename TT, typename TO>
+__global__ void gated_side_kernel(const float* __restrict__ z, const TT* __restrict__ table, const int32_t* __restrict__ ids,
+                                  TO* __restrict__ out, int width, int ds, int table_cols, int first, int vocab, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int t = static_cast<int>(i / width), c = static_cast<int>(i % width);
+    float v = 0.f;
+    const int id = ids[t];
+    if (c < ds && id >= 0 && id < vocab)
+        v = gelu_tanh_f(z[i]) * ld(table + static_cast<size_t>(id) * table_cols + first + c);
+    st(out + i, v);
+}
+
+NI_EXPORT int ni_gated_side(const void* z, const void* table, const void* ids, void* out, int T, int width, int ds,
+                            int table_cols, int first, int vocab, int dtype, hipStream_t stream) {
+    const size_t n = static_cast<size_t>(T) * width;
+    if (n == 0) return 0;
+    if (dtype == 0)
+        gated_side_kernel<float, float><<<blocks_of(n, 256), 256, 0, stream>>>(
+            (const float*)z, (const float*)table, (const int32_t*)ids, (float*)out, width, ds, table_cols, first, vocab, n);
+    else
+        gated_side_kernel<bf16_t, bf16_t><<<blocks_of(n, 256), 256, 0, stream>>>(
+            (const float*)z, (const bf16_t*)table, (const int32_t*)ids, (bf16_t*)out, width, ds, table_cols, first, vocab, n);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- h += y / sqrt(mean(y^2) + eps) * w
+__global__ void add_rmsnormed_kernel(float* __restrict__ h, const float* __restrict__ y, const float* __restrict__ w,
+                                     int d, float eps) {
+    __shared__ float scratch[16];
+    const size_t base = static_cast<size_t>(blockIdx.x) * d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = y[base + i];
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) h[base + i] += (y[base + i] * inv) * w[i];
+}
+
+NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int d, float eps, hipStream_t stream) {
+    if (T <= 0) return 0;
+    const int threads = d <= 256 ? 64 : d <= 1024 ? 256 : 512;
+    add_rmsnormed_kernel<<<T, threads, 0, stream>>>((float*)h, (const float*)y, (const float*)w, d, eps);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- the router's choice
+// z float32 [T, E]: the `top` largest logits of a row (the lower index on equal logits), their softmax
+// among themselves.  chosen int32 [T, top], mix float32 [T, top], and (if asked for) the same as a row
+// over all experts, zero where an expert was not chosen.
+__global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen, float* __restrict__ mix,
+                                 float* __restrict__ mix_all, int T, int E, int top) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) return;
+    const float* row = z + static_cast<size_t>(t) * E;
+    int32_t* c = chosen + static_cast<size_t>(t) * top;
+    float* m = mix + static_cast<size_t>(t) * top;
+    float best = 0.f, total = 0.f;
+    for (int k = 0; k < top; ++k) {
+        int at = -1;
+        float v = 0.f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= (c[j] == e);
+            const float ze = row[e];
+            if (!taken && (at < 0 || ze > v)) { at = e; v = ze; }
+        }
+        c[k] = at;
+        if (k == 0) best = v;
+        const float w = expf(v - best);
+        m[k] = w;
+        total += w;
+    }
+    if (mix_all)
+        for (int e = 0; e < E; ++e) mix_all[static_cast<size_t>(t) * E + e] = 0.f;
+    for (int k = 0; k < top; ++k) {
+        const float w = m[k] / total;
+        m[k] = w;
+        if (mix_all) mix_all[static_cast<size_t>(t) * E + c[k]] = w;
+    }
+}
+
+NI_EXPORT int ni_route_top(const void* z, void* chosen, void* mix, void* mix_all, int T, int E, int top, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (top < 1 || top > E) return -1;
+    route_top_kernel<<<blocks_of(T, 64), 64, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- all experts at once, for many rows
+// act[t, e * ff + i] = mix_all[t, e] * relu(up[t, e * ff + i])^2 : an expert that was not chosen gives
+// zeros, and the product with the experts' down matrices laid side by side is the weighted sum.
+template <typename T>
+__global__ void experts_act_kernel(const T* __restrict__ up, const float* __restrict__ mix_all, T* __restrict__ act,
+                                   int E, int ff, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t width = static_cast<size_t>(E) * ff;
+    const size_t t = i / width;
+    const int e = static_cast<int>((i % width) / ff);
+    const float w = mix_all[t * E + e];
+    float v = 0.f;
+    if (w != 0.f) {
+        const float u = fmaxf(ld(up + i), 0.f);
+        v = w * (u * u);
+    }
+    st(act + i, v);
+}
+
+NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int dtype, hipStream_t stream) {
+    const size_t n = static_cast<size_t>(T) * E * ff;
+    if (n == 0) return 0;
+    if (dtype == 0)
+        experts_act_kernel<float><<<blocks_of(n, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, n);
+    else
+        experts_act_kernel<bf16_t><<<blocks_of(n, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, n);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- the chosen experts alone, for few rows
+// Only the matrices of the chosen experts are read, each row of a matrix by one wavefront: its lanes
+// take neighbouring pieces of the row, so a row streams from memory in whole lines.
+//   hid[t * top + k, i] = relu(W_up[chosen[t, k] * ff + i, :] . x[t, :])^2        (float32)
+//   out[t, r] = sum_k mix[t, k] * W_down[r, chosen[t, k] * ff : +ff] . hid[t * top + k, :]
+template <typename T>
+__global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restrict__ w_up, const int32_t* __restrict__ chosen,
+                                      float* __restrict__ hid, int d, int ff, int top, int rows_per_block) {
+    const int pair = blockIdx.x;                 // t * top + k
+    const int t = pair / top;
+    const int e = chosen[pair];
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
+    const T* xr = x + static_cast<size_t>(t) * d;
+    const int first = blockIdx.y * rows_per_block;
+    for (int i = first + wave; i < first + rows_per_block && i < ff; i += waves) {
+        const T* wr = w_up + (static_cast<size_t>(e) * ff + i) * d;
+        float s = 0.f;
+        for (int c = lane; c < d; c += WAVE) s += ld(wr + c) * ld(xr + c);
+        s = wave_sum(s);
+        if (lane == 0) {
+            const float u = fmaxf(s, 0.f);
+            hid[static_cast<size_t>(pair) * ff + i] = u * u;
+        }
+    }
+}
+
+template <typename T>
+__global__ void experts_down_few_kernel(const float* __restrict__ hid, const T* __restrict__ w_down,
+                                        const int32_t* __restrict__ chosen, const float* __restrict__ mix,
+                                        float* __restrict__ out, int d, int ff, int E, int top, int rows_per_block) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
+    const int first = blockIdx.y * rows_per_block;
+    const size_t row_stride = static_cast<size_t>(E) * ff;
+    for (int r = first + wave; r < first + rows_per_block && r < d; r += waves) {
+        float total = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int e = chosen[t * top + k];
+            const T* wr = w_down + static_cast<size_t>(r) * row_stride + static_cast<size_t>(e) * ff;
+            const float* hr = hid + (static_cast<size_t>(t) * top + k) * ff;
+            float s = 0.f;
+            for (int c = lane; c < ff; c += WAVE) s += ld(wr + c) * hr[c];
+            total += mix[t * top + k] * wave_sum(s);
+        }
+        if (lane == 0) out[static_cast<size_t>(t) * d + r] = total;
+    }
+}
+
+NI_EXPORT int ni_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
+                             void* hid, void* out, int T, int d, int ff, int E, int top, int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    const int rows = 16;
+    dim3 g1(T * top, (ff + rows - 1) / rows), g2(T, (d + rows - 1) / rows);
+    if (dtype == 0) {
+        experts_up_few_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)w_up, (const int32_t*)chosen,
+                                                             (float*)hid, d, ff, top, rows);
+        experts_down_few_kernel<float><<<g2, 256, 0, stream>>>((const float*)hid, (const float*)w_down, (const int32_t*)chosen,
+                                                               (const float*)mix, (float*)out, d, ff, E, top, rows);
+    } else {
+        experts_up_few_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w_up, (const int32_t*)chosen,
+                                                              (float*)hid, d, ff, top, rows);
+        experts_down_few_kernel<bf16_t><<<g2, 256, 0, stream>>>((const float*)hid, (const bf16_t*)w_down, (const int32_t*)chosen,
+                                                                (const float*)mix, (float*)out, d, ff, E, top, rows);
+    }
+    return NI_LAUNCH_RESULT();
+}

@@ -24,10 +24,16 @@ class Model:
         self.embedding = build_part("embedding", spec.embedding, tensors, rt)
         self.blocks = [get_part("block", b.kind)(b, tensors, rt) for b in spec.blocks]
         self.final_norm = build_part("norm", spec.final_norm, tensors, rt)
+        self.pass_input = None if spec.pass_input is None else build_part("pass_input", spec.pass_input, tensors, rt)
+        # a function (index of the entry of the order, h) called after every entry with the complete residual
+        # stream, for whoever wants to look at a pass layer by layer; None costs nothing
+        self.tap = None
         self.head = build_part("head", spec.head, tensors, rt)
         for run in spec.order:
             if not 0 <= run.block < len(self.blocks):
                 raise ValueError(f"the order names block {run.block}, the model has {len(self.blocks)}")
+            if run.enter is not None and self.pass_input is None:
+                raise ValueError(f"an entry of the order adds row {run.enter} of a pass input, the model has none")
         self._needs: Dict[int, CacheNeed] = {}
         writers = set()
         for run in spec.order:
@@ -43,7 +49,8 @@ class Model:
         self.max_positions = spec.max_positions
 
     def _all_parts(self):
-        return [self.embedding, self.final_norm, self.head] + list(self.blocks)
+        return [self.embedding, self.final_norm, self.head] + list(self.blocks) + \
+            ([] if self.pass_input is None else [self.pass_input])
 
     def graph_safe(self) -> bool:
         """Whether a step of this model may be recorded into a HIP graph: every part says of itself
@@ -54,6 +61,11 @@ class Model:
         """Whether running the same step twice leaves the caches as running it once does: true of keys
         and values written to their places, not of a per-request state that a part updates in place."""
         return all(flag_of(p, "idempotent", True) for p in self._all_parts())
+
+    def _settled(self, h, pending):
+        """A copy of the stream with what is pending added (for :attr:`tap`; the pass itself goes on as it was)."""
+        pending = pending_for(None, pending, self.rt.dtype)
+        return h.clone() if pending is None else h + pending.to(h.dtype)
 
     def cache_needs(self) -> Dict[int, CacheNeed]:
         return dict(self._needs)
@@ -71,6 +83,11 @@ class Model:
         for i, run in enumerate(order):
             cache: LayerCache = layer_cache(run.cache, run.writes_cache)
             block = self.blocks[run.block]
+            if run.enter is not None:
+                if pending is not None:        # the stream has to be complete before a row is added to it
+                    h = self.pass_input.settle(h, pending_for(None, pending, self.rt.dtype))
+                    pending = None
+                h = self.pass_input.forward(h, run.enter)
             # what the block behind this one would like to find beside the stream (its first norm's input half
             # done by this block's last product), if both blocks know of that
             wants = getattr(self.blocks[order[i + 1].block], "wants_scaled", None) if i + 1 < len(order) else None
@@ -79,6 +96,8 @@ class Model:
                 h, pending = block.forward(h, pending, ctx, cache, leave=leave)
             else:
                 h, pending = block.forward(h, pending, ctx, cache)
+            if self.tap is not None:
+                self.tap(i, h if pending is None else self._settled(h, pending))
         if ctx.logit_rows is None or ctx.logit_rows.shape[0] == 0:
             return None
         x = self.final_norm.forward(h, pending_for(self.final_norm, pending, self.rt.dtype), rows=ctx.logit_rows)

@@ -24,7 +24,7 @@ def parse_args(argv: List[str]):
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time; the page pool is made for this many")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (default 16)")
-    ap.add_argument("--max-requests", type=int, default=16, help="most requests live at a time (default 16)")
+    ap.add_argument("--max-requests", type=int, default=4, help="most requests live at a time: the state slots (default 4)")
     return ap.parse_args(argv)
 
 

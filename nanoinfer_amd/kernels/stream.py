@@ -1,0 +1,250 @@
+"""Python face of the kernels in ``csrc/stream_ops.hip``, ``csrc/delta_rule.hip`` and
+``csrc/bias_attention.hip``: sums onto the residual stream, a scaled embedding with position rows, a
+token's side input, the router and its experts, the gated delta rule, and attention with a bias by
+distance.  Shapes, types and devices are checked here, on the host, before a kernel is launched.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from ..csrc import build as _build
+from . import KernelError, _check, _gpu, _load, _need, _ptr, _stream, dtype_code
+
+
+def stream_lib() -> ctypes.CDLL:
+    return _load(_build.STREAM_OPS)
+
+
+def bias_attention_lib() -> ctypes.CDLL:
+    return _load(_build.BIAS_ATTENTION)
+
+
+def delta_rule_lib(key_size: int) -> ctypes.CDLL:
+    return _load(_build.delta_rule_target(key_size))
+
+
+_size_t = ctypes.c_size_t
+_float = ctypes.c_float
+
+
+# ------------------------------------------------------------------ the residual stream
+
+def embed_scaled(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, pos_table: Optional[torch.Tensor],
+                 scale: float, out: torch.Tensor) -> torch.Tensor:
+    """``out[t] = table[ids[t]] * scale + pos_table[positions[t]]`` as float32 (no position rows: the first term)."""
+    T = ids.shape[0]
+    vocab, d = table.shape
+    _gpu(ids, "ids", torch.int32, (T,))
+    _gpu(positions, "positions", torch.int32, (T,))
+    _gpu(table, "table")
+    _gpu(out, "out", torch.float32, (T, d))
+    max_pos = 0
+    if pos_table is not None:
+        max_pos = pos_table.shape[0]
+        _gpu(pos_table, "pos_table", table.dtype, (max_pos, d))
+    _check(stream_lib().ni_embed_scaled(_ptr(ids), _ptr(positions), _ptr(table), _ptr(pos_table), _ptr(out), T, d, vocab,
+                                        max_pos, _float(scale), dtype_code(table.dtype), _stream()), "embed_scaled")
+    return out
+
+
+def add_vector(h: torch.Tensor, vec: torch.Tensor) -> torch.Tensor:
+    """``h[t] += vec`` for every row of the float32 stream."""
+    T, d = h.shape
+    _gpu(h, "h", torch.float32)
+    _gpu(vec, "vec", torch.float32, (d,))
+    _check(stream_lib().ni_add_vector(_ptr(h), _ptr(vec), T, d, _stream()), "add_vector")
+    return h
+
+
+def stream_add(h: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None,
+               x_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``h += (a + b)`` in float32 (``b`` may be absent); ``x_out``, if given, takes the new stream in its own
+    type.  ``a`` and ``b`` are float32 or bfloat16 [T, d]."""
+    T, d = h.shape
+    _gpu(h, "h", torch.float32)
+    _gpu(a, "a", None, (T, d))
+    if b is not None:
+        _gpu(b, "b", None, (T, d))
+    if x_out is not None:
+        _gpu(x_out, "x_out", None, (T, d))
+    _check(stream_lib().ni_stream_add(_ptr(h), _ptr(a), dtype_code(a.dtype), _ptr(b), dtype_code(b.dtype) if b is not None else 0,
+                                      _ptr(x_out), dtype_code(x_out.dtype) if x_out is not None else 0, T, d, _stream()),
+           "stream_add")
+    return h
+
+
+def gated_side(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, first: int, size: int, out: torch.Tensor) -> torch.Tensor:
+    """``out[t, c] = gelu_tanh(z[t, c]) * table[ids[t], first + c]`` for c < size, zero in the padding columns."""
+    T, width = z.shape
+    vocab, cols = table.shape
+    _gpu(z, "z", torch.float32)
+    _gpu(table, "table")
+    _gpu(ids, "ids", torch.int32, (T,))
+    _gpu(out, "out", table.dtype, (T, width))
+    _need(0 <= first and first + size <= cols and size <= width, "the side rows do not lie inside the table")
+    _check(stream_lib().ni_gated_side(_ptr(z), _ptr(table), _ptr(ids), _ptr(out), T, width, size, cols, first, vocab,
+                                      dtype_code(table.dtype), _stream()), "gated_side")
+    return out
+
+
+def add_rmsnormed(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``h += y / sqrt(mean(y^2) + eps) * weight`` row by row, all float32."""
+    T, d = h.shape
+    _gpu(h, "h", torch.float32)
+    _gpu(y, "y", torch.float32, (T, d))
+    _gpu(weight, "weight", torch.float32, (d,))
+    _check(stream_lib().ni_add_rmsnormed(_ptr(h), _ptr(y), _ptr(weight), T, d, _float(eps), _stream()), "add_rmsnormed")
+    return h
+
+
+# ------------------------------------------------------------------ router and experts
+
+def route_top(z: torch.Tensor, top: int, mix_all: bool):
+    """The ``top`` largest logits of every row of ``z`` float32 [T, E] and their softmax among themselves:
+    ``(chosen int32 [T, top], mix float32 [T, top], mix over all experts float32 [T, E] or None)``."""
+    T, E = z.shape
+    _gpu(z, "z", torch.float32)
+    _need(1 <= top <= E, f"{top} of {E} experts cannot be chosen")
+    chosen = torch.empty(T, top, dtype=torch.int32, device=z.device)
+    mix = torch.empty(T, top, dtype=torch.float32, device=z.device)
+    dense = torch.empty(T, E, dtype=torch.float32, device=z.device) if mix_all else None
+    _check(stream_lib().ni_route_top(_ptr(z), _ptr(chosen), _ptr(mix), _ptr(dense), T, E, top, _stream()), "route_top")
+    return chosen, mix, dense
+
+
+def experts_act(up: torch.Tensor, mix_all: torch.Tensor, ff: int) -> torch.Tensor:
+    """``mix_all[t, e] * relu(up[t, e * ff + i])^2`` in the type of ``up``."""
+    T, width = up.shape
+    E = mix_all.shape[1]
+    _gpu(up, "up")
+    _gpu(mix_all, "mix_all", torch.float32, (T, E))
+    _need(width == E * ff, "the experts' hidden rows do not match the router")
+    act = torch.empty_like(up)
+    _check(stream_lib().ni_experts_act(_ptr(up), _ptr(mix_all), _ptr(act), T, E, ff, dtype_code(up.dtype), _stream()), "experts_act")
+    return act
+
+
+EXPERTS_FEW_ROWS = 16       # up to here only the chosen experts' matrices are read, row by row
+
+
+def experts_few(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor, mix: torch.Tensor,
+                ff: int) -> torch.Tensor:
+    """The weighted sum of the chosen experts for a few rows: ``w_up`` [E * ff, d], ``w_down`` [d, E * ff];
+    returns float32 [T, d]."""
+    T, d = x.shape
+    top = chosen.shape[1]
+    E = w_up.shape[0] // ff
+    _gpu(x, "x", w_up.dtype)
+    _gpu(w_up, "w_up", None, (E * ff, d))
+    _gpu(w_down, "w_down", w_up.dtype, (d, E * ff))
+    _gpu(chosen, "chosen", torch.int32, (T, top))
+    _gpu(mix, "mix", torch.float32, (T, top))
+    hid = torch.empty(T * top, ff, dtype=torch.float32, device=x.device)
+    out = torch.empty(T, d, dtype=torch.float32, device=x.device)
+    _check(stream_lib().ni_experts_few(_ptr(x), _ptr(w_up), _ptr(w_down), _ptr(chosen), _ptr(mix), _ptr(hid), _ptr(out),
+                                       T, d, ff, E, top, dtype_code(x.dtype), _stream()), "experts_few")
+    return out
+
+
+# ------------------------------------------------------------------ gated delta rule
+
+def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+               norm_w: torch.Tensor, state: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor,
+               q_len: torch.Tensor, state_slot: torch.Tensor, G: int, H: int, dk: int, dv: int, taps: int, eps: float,
+               out_dtype: torch.dtype) -> torch.Tensor:
+    """One step of the gated delta rule with a decay per key channel for all sequences of the step.
+
+    ``proj`` float32 [T, >= C + H] holds q [G*dk] | k [G*dk] | v [H*dv] | b [H] as projected (C the first
+    three); ``low`` float32 [T, H*dk + H*dv] the decay's and the output gate's pre-activations; ``conv``
+    float32 [C, taps]; ``state`` float32 [slots, H*dv*dk + (taps-1)*C]: the memory of every head (stored
+    [head, value channel, key channel]) and the convolutions' last inputs, both moved on by this call.
+    Returns the normalised, gated read-out [T, H*dv] in ``out_dtype``."""
+    T, proj_cols = proj.shape
+    B = q_start.shape[0]
+    C = 2 * G * dk + H * dv
+    _gpu(proj, "proj", torch.float32)
+    _need(proj_cols >= C + H, "proj is too narrow")
+    _gpu(low, "low", torch.float32, (T, H * dk + H * dv))
+    _gpu(conv, "conv", torch.float32, (C, taps))
+    _gpu(a_log, "a_log", torch.float32, (H,))
+    _gpu(dt_bias, "dt_bias", torch.float32, (H * dk,))
+    _gpu(norm_w, "norm_w", torch.float32, (dv,))
+    _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous(), "state must be float32 [slots, n] on the GPU")
+    conv_off = H * dv * dk
+    _need(state.shape[1] == conv_off + (taps - 1) * C, "state has the wrong size")
+    _gpu(seq_of_token, "seq_of_token", torch.int32, (T,))
+    for name, t in (("q_start", q_start), ("q_len", q_len), ("state_slot", state_slot)):
+        _need(t.is_cuda and t.dtype == torch.int32 and t.shape == (B,), f"{name} must be int32 [{B}] on the GPU")
+    _need(H % G == 0 and taps >= 1, "heads and taps")
+    lib = delta_rule_lib(dk)
+    prep = torch.empty(T, C + H + H * dk + H * dv, dtype=torch.float32, device=proj.device)
+    stride = state.shape[1]
+    _check(lib.ni_delta_prepare(_ptr(proj), _ptr(low), _ptr(conv), _ptr(a_log), _ptr(dt_bias), _ptr(state), _ptr(seq_of_token),
+                                _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(prep), T, B, G, H, dk, dv, taps, proj_cols,
+                                _size_t(stride), _size_t(conv_off), _stream()), "delta_prepare")
+    o = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
+    y = torch.empty(T, H * dv, dtype=out_dtype, device=proj.device)
+    _check(lib.ni_delta_rule(_ptr(prep), _ptr(state), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(o), _ptr(norm_w),
+                             _ptr(y), T, B, G, H, dk, dv, _float(eps), _size_t(stride), dtype_code(out_dtype), _stream()),
+           "delta_rule")
+    return y
+
+
+# ------------------------------------------------------------------ attention with a bias by distance
+
+def bias_attention_rows() -> int:
+    """Rows of (token, head) that one workgroup of the kernel takes."""
+    return 16
+
+
+def kv_store(qkv: torch.Tensor, k_off: int, v_off: int, slot_mapping: torch.Tensor, kpool: torch.Tensor,
+             vpool: torch.Tensor) -> None:
+    """Keys (columns from ``k_off``) and values (from ``v_off``) of the rows of ``qkv`` into their page slots."""
+    T, width = qkv.shape
+    pages, G, ps, dk = kpool.shape
+    dv = vpool.shape[3]
+    _gpu(qkv, "qkv")
+    _gpu(kpool, "kpool", qkv.dtype)
+    _gpu(vpool, "vpool", qkv.dtype, (pages, G, ps, dv))
+    _gpu(slot_mapping, "slot_mapping", torch.int32, (T,))
+    _need(k_off + G * dk <= width and v_off + G * dv <= width, "keys or values lie outside the rows")
+    _check(bias_attention_lib().ni_kv_store(_ptr(qkv), width, k_off, v_off, _ptr(slot_mapping), _ptr(kpool), _ptr(vpool),
+                                            T, G, dk, dv, ps, dtype_code(qkv.dtype), _stream()), "kv_store")
+
+
+def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                   tiles: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int, scale: float,
+                   temp_coef: float, temp_every: int, heads_per_chunk: int) -> torch.Tensor:
+    """Causal attention of the query heads in the first ``H * dk`` columns of ``qkv`` over the paged cache.
+    ``tiles`` int32 [n, 4]: (sequence, first row, tokens, first position) with tokens * heads of a chunk <= 16;
+    ``bias`` float32 [distances, H] or None; ``out`` [T, H * dv]."""
+    T, width = qkv.shape
+    pages, G, ps, dk = kpool.shape
+    dv = vpool.shape[3]
+    _gpu(qkv, "qkv")
+    _gpu(kpool, "kpool", qkv.dtype)
+    _gpu(vpool, "vpool", qkv.dtype, (pages, G, ps, dv))
+    _need(block_table.is_cuda and block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be int32 [B, pages] on the GPU")
+    _need(tiles.is_cuda and tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
+          "tiles must be int32 [n, 4] on the GPU")
+    _gpu(out, "out", qkv.dtype, (T, H * dv))
+    _need(H % G == 0 and H * dk <= width, "heads")
+    distances = 0
+    if bias is not None:
+        distances = bias.shape[0]
+        _gpu(bias, "bias", torch.float32, (distances, H))
+        _need(distances >= 1, "an empty bias table")
+    _need(dv <= 256, "values of more than 256 channels are not compiled")
+    _need(1 <= heads_per_chunk <= 16, "heads_per_chunk")
+    err = bias_attention_lib().ni_bias_attention(_ptr(qkv), width, _ptr(kpool), _ptr(vpool), _ptr(block_table),
+                                                 block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(bias), distances,
+                                                 _ptr(out), H, G, dk, dv, ps, _float(scale), _float(temp_coef), int(temp_every),
+                                                 heads_per_chunk, dtype_code(qkv.dtype), _stream())
+    if err == -2:
+        raise KernelError(f"keys of {dk} and values of {dv} channels do not fit the kernel's staging memory")
+    _check(err, "bias_attention")
+    return out

@@ -8,7 +8,7 @@ The reference chooses a C++ class and an enum by a preset name in each demo
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, List
+from typing import Any, Callable, Dict, List, Optional
 
 from .config.spec import ModelSpec
 from .weights.random_init import InitRule
@@ -24,12 +24,15 @@ class Architecture:
     config_from_dict: Callable[[Dict[str, Any]], Any]   # config.json -> typed configuration
     build_spec: Callable[[Any], ModelSpec]               # typed configuration -> model as data
     init: InitRule = field(default_factory=InitRule)     # distribution of each tensor of the random-weights mode
+    # (typed configuration, tensor name -> shape of the checkpoint) -> typed configuration: for an architecture
+    # whose config.json leaves some sizes to the shapes of its tensors; None: config.json says everything
+    sizes_from_shapes: Optional[Callable[[Any, Dict[str, tuple]], Any]] = None
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}
 
 # one table per family of parts; a part class is looked up by the ``kind`` of its spec
-PART_FAMILIES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head")
+PART_FAMILIES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head", "token_input", "pass_input")
 PARTS: Dict[str, Dict[str, type]] = {family: {} for family in PART_FAMILIES}
 
 
@@ -74,6 +77,8 @@ def get_part(family: str, kind: str) -> type:
 
 def architecture_of(config_json: Dict[str, Any]) -> Architecture:
     archs = config_json.get("architectures")
+    if not archs and isinstance(config_json.get("architecture"), str):
+        archs = [config_json["architecture"]]         # some exporters name the one architecture as a string
     if not archs:
         raise RegistryError(f"config.json names no architecture; known: {sorted(ARCHITECTURES)}")
     return get_architecture(str(archs[0]))

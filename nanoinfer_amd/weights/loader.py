@@ -49,6 +49,8 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, Tuple[int, ...]]:
     requests = list(get_part("embedding", spec.embedding.kind).weight_requests(spec.embedding))
     for b in spec.blocks:
         requests += get_part("block", b.kind).weight_requests(b)
+    if spec.pass_input is not None:
+        requests += get_part("pass_input", spec.pass_input.kind).weight_requests(spec.pass_input)
     requests += get_part("norm", spec.final_norm.kind).weight_requests(spec.final_norm)
     requests += get_part("head", spec.head.kind).weight_requests(spec.head)
     out: Dict[str, Tuple[int, ...]] = {}
@@ -242,4 +244,7 @@ def read_model_folder(folder: str):
     raw = read_config_json(folder)
     arch = architecture_of(raw)
     cfg = arch.config_from_dict(raw)
+    if arch.sizes_from_shapes is not None:
+        ckpt = _Checkpoint(folder)
+        cfg = arch.sizes_from_shapes(cfg, {n: tuple(ckpt.shape(n)) for n in ckpt.names()})
     return arch, cfg, arch.build_spec(cfg)
