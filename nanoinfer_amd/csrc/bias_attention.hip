@@ -48,7 +48,7 @@ template <typename T>
 __global__ void __launch_bounds__(WAVES * WAVE)
 bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
                       const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
-                      const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
+                      const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
                       int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk) {
     extern __shared__ float lds[];
     const int dkp = dk + 1;                       // a lane reads its key's row: odd strides spread the banks
@@ -57,7 +57,10 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
     float* Vs = Ks + KEYS * dkp;                  // [KEYS][dv]
     float* Ps = Vs + KEYS * dv;                   // [WAVES][ROWS_PER_WAVE][KEYS]
     const int tile = blockIdx.x, g = blockIdx.y, chunk = blockIdx.z;
-    const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2], first_pos = tiles[4 * tile + 3];
+    // the first position is read from the step's positions, not from the tile: a recorded decode step is replayed
+    // with new positions and the tiles it was recorded with
+    const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2];
+    const int first_pos = positions[first_row];
     const int group = H / G;
     const int heads_here = std::min(heads_per_chunk, group - chunk * heads_per_chunk);
     const int head0 = g * group + chunk * heads_per_chunk;
@@ -190,7 +193,7 @@ NI_EXPORT int ni_kv_store(const void* qkv, int row_stride, int k_off, int v_off,
 NI_EXPORT int ni_bias_attention_rows() { return ROWS; }
 
 NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
-                                int table_width, const void* tiles, int n_tiles, const void* bias, int distances, void* out,
+                                int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias, int distances, void* out,
                                 int H, int G, int dk, int dv, int page_size, float scale, float temp_coef, int temp_every,
                                 int heads_per_chunk, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
@@ -208,7 +211,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         if (err != hipSuccess) return (int)err;
         bias_attention_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
-            (const int32_t*)tiles, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
+            (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
             temp_every, heads_per_chunk);
     } else {
         static size_t allowed = 48 * 1024;
@@ -217,7 +220,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         if (err != hipSuccess) return (int)err;
         bias_attention_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
-            (const int32_t*)tiles, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
+            (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
             temp_every, heads_per_chunk);
     }
     return NI_LAUNCH_RESULT();

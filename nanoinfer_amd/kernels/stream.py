@@ -216,10 +216,11 @@ def kv_store(qkv: torch.Tensor, k_off: int, v_off: int, slot_mapping: torch.Tens
 
 
 def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
-                   tiles: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int, scale: float,
+                   tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int, scale: float,
                    temp_coef: float, temp_every: int, heads_per_chunk: int) -> torch.Tensor:
     """Causal attention of the query heads in the first ``H * dk`` columns of ``qkv`` over the paged cache.
-    ``tiles`` int32 [n, 4]: (sequence, first row, tokens, first position) with tokens * heads of a chunk <= 16;
+    ``tiles`` int32 [n, 4]: (sequence, first row, tokens, -) with tokens * heads of a chunk <= 16, the tokens of a
+    tile being consecutive ones of one sequence; ``positions`` int32 [T] the position of every row;
     ``bias`` float32 [distances, H] or None; ``out`` [T, H * dv]."""
     T, width = qkv.shape
     pages, G, ps, dk = kpool.shape
@@ -232,6 +233,7 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _need(tiles.is_cuda and tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
           "tiles must be int32 [n, 4] on the GPU")
     _gpu(out, "out", qkv.dtype, (T, H * dv))
+    _gpu(positions, "positions", torch.int32, (T,))
     _need(H % G == 0 and H * dk <= width, "heads")
     distances = 0
     if bias is not None:
@@ -241,7 +243,7 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _need(dv <= 256, "values of more than 256 channels are not compiled")
     _need(1 <= heads_per_chunk <= 16, "heads_per_chunk")
     err = bias_attention_lib().ni_bias_attention(_ptr(qkv), width, _ptr(kpool), _ptr(vpool), _ptr(block_table),
-                                                 block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(bias), distances,
+                                                 block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions), _ptr(bias), distances,
                                                  _ptr(out), H, G, dk, dv, ps, _float(scale), _float(temp_coef), int(temp_every),
                                                  heads_per_chunk, dtype_code(qkv.dtype), _stream())
     if err == -2:

@@ -210,7 +210,7 @@ class BiasAttention(Part):
         if tiles is None:
             raise K.KernelError("this step was recorded without the tiles of its tokens")
         out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
-        K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, self.bias, out, self.H, self.scale,
+        K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H, self.scale,
                          self.temp_coef, self.temp_every, self.heads_per_chunk)
         return K.linear(out, self.w_o, out_dtype=torch.float32)
 
