@@ -1,0 +1,325 @@
+"""Zekalorn through the engine against the plain implementation (``plain_zekalorn.py``): every mechanism
+alone and all together, whole prompts against portions and single tokens, unequal batches against each
+request alone, pages and state slots that are used again, keys far back and at the edges of pages and of
+the attention kernel's runs of 64 keys, long decoding, and greedy generation through ``Engine``.
+
+Models are written with the random-weights mode in bfloat16 (so that both compute types see the same
+numbers as the plain implementation) with larger matrices than the architecture's rule draws, so that a
+mixer or feed-forward that went wrong moves the logits by far more than the tolerance; where random
+weights would still hide a fault (one far key among hundreds) the test sets the tensors that show it.
+"""
+import functools
+import os
+import random
+import shutil
+import tempfile
+
+import pytest
+import torch
+
+import plain_zekalorn as P
+import zekalorn_configs as Z
+from gpu_common import assert_close, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+_root = None
+_folders = {}
+
+
+def folder_of(name: str, seed: int = 11, edit=None) -> str:
+    """A model folder for configuration ``name``; ``edit(tensors)`` may change tensors before they are written."""
+    global _root
+    key = (name, seed, None if edit is None else edit.__name__)
+    if key not in _folders:
+        import nanoinfer_amd  # noqa: F401
+        from nanoinfer_amd.weights.loader import make_random_model, write_model_folder
+        if _root is None:
+            _root = tempfile.mkdtemp(prefix="zekalorn-tests-")
+            import atexit
+            atexit.register(shutil.rmtree, _root, ignore_errors=True)
+        path = make_random_model(os.path.join(_root, f"{name}-{seed}-{len(_folders)}"), Z.ALL[name], seed, dtype="bfloat16",
+                                 matrix_std=0.12)
+        if edit is not None:
+            config, tensors = P.read_model_folder(path)
+            edit(tensors)
+            write_model_folder(path, config, {k: v.contiguous() for k, v in tensors.items()})
+        _folders[key] = path
+    return _folders[key]
+
+
+@functools.lru_cache(maxsize=None)
+def plain(folder: str, tokens: tuple) -> torch.Tensor:
+    config, tensors = P.read_model_folder(folder)
+    return P.forward(config, tensors, list(tokens))
+
+
+def runner_for(folder, dtype, **kw):
+    from nanoinfer_amd.engine.runner import ModelRunner
+    kw.setdefault("page_size", 8)
+    kw.setdefault("max_tokens", 2048)
+    kw.setdefault("max_requests", 4)
+    return ModelRunner(folder, dtype=dtype, **kw)
+
+
+def replay(runner, requests, steps):
+    """Run ``steps`` (each a dict request -> number of its next tokens), asking for every row; returns
+    request -> logits [tokens, vocab].  A request ends with its last token."""
+    from nanoinfer_amd.engine.runner import StepEntry
+    done = {r: 0 for r in requests}
+    rows = {r: [] for r in requests}
+    for counts in steps:
+        entries = [StepEntry(r, list(requests[r][done[r]:done[r] + c]), list(range(c))) for r, c in counts.items()]
+        out = runner.step(entries, end=[r for r, c in counts.items() if done[r] + c == len(requests[r])])
+        at = 0
+        for r, c in counts.items():
+            rows[r].append(out[at:at + c].clone())
+            at += c
+            done[r] += c
+    assert all(done[r] == len(requests[r]) for r in requests)
+    return {r: torch.cat(v) for r, v in rows.items()}
+
+
+def cuts(n, sizes):
+    """``n`` tokens cut into portions of the given sizes in turn."""
+    out, i = [], 0
+    while n > 0:
+        c = min(n, sizes[i % len(sizes)])
+        out.append(c)
+        n -= c
+        i += 1
+    return out
+
+
+DTYPES = ["float32", "bfloat16"]
+
+
+# ------------------------------------------------------------------ every mechanism alone
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["attention_only", "attention_plain", "delta_only", "delta_no_conv", "dense_ff",
+                                  "routed_ff", "side_input"])
+def test_one_mechanism_whole_prompt_and_token_by_token(name, dtype):
+    """A model of one layer with one mechanism switched on: a whole prompt, then the same tokens as a short
+    portion followed by single tokens, both equal to the plain implementation row by row."""
+    folder = folder_of(name)
+    toks = random_tokens(Z.ALL[name]["vocab"], 75, 5)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype)
+    got = replay(runner, {"w": toks}, [{"w": len(toks)}])["w"]
+    assert_close(got, want, dtype, f"{name} whole")
+    got = replay(runner, {"d": toks}, [{"d": 3}] + [{"d": 1}] * (len(toks) - 3))["d"]
+    assert_close(got, want, dtype, f"{name} token by token")
+    assert not runner.cache.live_requests()
+
+
+@pytest.mark.parametrize("name", ["attention_only", "delta_only", "routed_ff", "side_input"])
+def test_the_mechanism_matters_in_these_models(name):
+    """The comparisons above would pass with a mechanism that does nothing if it weighed nothing: with its
+    output matrix at zero the plain logits move by hundreds of times the float32 tolerance."""
+    folder = folder_of(name)
+    config, tensors = P.read_model_folder(folder)
+    toks = list(random_tokens(config["vocab"], 40, 5))
+    want = P.forward(config, tensors, toks)
+    dead = dict(tensors)
+    for key in {"attention_only": ["l0.mix.o"], "delta_only": ["l0.mix.o"], "side_input": ["l0.side.proj"],
+                "routed_ff": [k for k in tensors if k.startswith("l0.mlp.e") and k.endswith(".down")]}[name]:
+        dead[key] = torch.zeros_like(tensors[key])
+    if name == "side_input":       # a zero before the norm is no input at all only with the norm's weight at zero too
+        dead["l0.side.norm"] = torch.zeros_like(tensors["l0.side.norm"])
+    diff = float((P.forward(config, dead, toks) - want).abs().max() / want.abs().max())
+    assert diff > 5e-3, diff
+
+
+# ------------------------------------------------------------------ the whole design, every schedule
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["mixed", "loop_all"])
+def test_portions_of_several_sizes_down_to_two_tokens(name, dtype):
+    folder = folder_of(name)
+    toks = random_tokens(Z.ALL[name]["vocab"], 150, 21)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype)
+    for sizes in ([150], [2], [37, 2, 23, 3], [64, 1, 1, 17], [5, 8, 16, 1]):
+        got = replay(runner, {"p": toks}, [{"p": c} for c in cuts(len(toks), sizes)])["p"]
+        assert_close(got, want, dtype, f"{name} in portions of {sizes}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("graphs", [True, False])
+def test_unequal_requests_in_one_batch_equal_each_alone_and_slots_are_used_again(dtype, graphs):
+    """Six requests of 1 to 130 tokens through a pool that holds three at a time and too few pages for all:
+    portions beside single tokens, requests that pause for a step, pages and state slots that the next
+    request takes over as they are.  Every row equals the plain implementation of its request alone."""
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    lengths = {"a": 130, "b": 1, "c": 47, "d": 80, "e": 2, "f": 66}
+    requests = {r: random_tokens(vocab, n, 40 + i) for i, (r, n) in enumerate(lengths.items())}
+    runner = runner_for(folder, dtype, max_tokens=8 * 36, max_requests=3, use_graphs=graphs)
+    steps = [{"a": 30}, {"a": 29, "b": 1, "c": 2}, {"a": 1, "c": 16}, {"c": 1, "a": 7}, {"a": 1, "c": 1}, {"a": 1, "c": 27},
+             {"a": 61, "c": 1}]
+    # c has ended; d and e come in on its pages and slot
+    steps += [{"d": 40, "e": 1}, {"e": 1, "d": 1}, {"d": 39}]
+    steps += [{"f": 64}, {"f": 1}, {"f": 1}]
+    got = replay(runner, requests, steps)
+    for r, toks in requests.items():
+        assert_close(got[r], plain(folder, toks), dtype, f"request {r}")
+    runner.cache.check()
+    assert not runner.cache.live_requests() and runner.cache.free_pages() == runner.cache.num_pages
+    assert runner.cache.slots.num_free == 3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_in_a_batch_of_recorded_steps(dtype):
+    """Three requests decode 140 tokens each side by side after prompts of unequal length, across many page
+    edges and two edges of the attention's runs of 64 keys, in recorded steps."""
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    prompts = {"x": 5, "y": 61, "z": 30}
+    requests = {r: random_tokens(vocab, n + 140, 70 + i) for i, (r, n) in enumerate(prompts.items())}
+    runner = runner_for(folder, dtype)
+    got = replay(runner, requests, [dict(prompts)] + [{r: 1 for r in prompts}] * 140)
+    assert any(key[0] == "d" for key in runner._recorded), "the decode steps were not recorded"
+    for r, toks in requests.items():
+        assert_close(got[r], plain(folder, toks), dtype, f"request {r}")
+
+
+# ------------------------------------------------------------------ far keys and edges
+
+def _far_sighted(tensors):
+    """One head looks as far back as it can (the bias of the last rows of its table is large), another at its
+    nearest neighbours; scores are sharp, so that a key that is missed or taken twice moves the output."""
+    rel = tensors["l0.mix.rel"].float()
+    rel[:] = 0.0
+    rel[-3:, 0] = 9.0
+    rel[:2, 1] = 9.0
+    tensors["l0.mix.rel"] = rel.to(torch.bfloat16)
+    for k in ("l0.mix.q", "l0.mix.k", "l0.mix.v", "l0.mix.o"):
+        tensors[k] = (tensors[k].float() * 2.5).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_keys_and_edges_of_pages_and_key_runs(dtype):
+    """A head whose bias prefers the farthest keys and sharp scores: prompts that end, portions that start and
+    single tokens that fall just before, on and just behind the edges of pages (8) and of the kernel's runs of
+    64 keys, over a few hundred keys."""
+    name = "attention_only"
+    folder = folder_of(name, edit=_far_sighted)
+    toks = random_tokens(Z.ALL[name]["vocab"], 330, 9)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype)
+    for first in (63, 64, 65, 127, 128, 129, 7, 8, 9, 255, 257):
+        rest = len(toks) - first
+        steps = [{"k": first}] + [{"k": 1}] * 3 + [{"k": c} for c in cuts(rest - 3, [62, 2, 1, 64, 3])]
+        got = replay(runner, {"k": toks}, steps)["k"]
+        assert_close(got, want, dtype, f"first portion of {first}")
+    # the far head does depend on the far keys: with the last rows of its bias gone the logits move
+    config, tensors = P.read_model_folder(folder)
+    tensors["l0.mix.rel"] = tensors["l0.mix.rel"].clone()
+    tensors["l0.mix.rel"][-3:, 0] = 0
+    assert float((P.forward(config, tensors, list(toks[:200]))[-1] - want[199]).abs().max() / want[199].abs().max()) > 1e-2
+
+
+def test_distance_rows_are_the_plain_buckets():
+    from nanoinfer_amd.parts.hybrid import distance_rows
+    for rows, far, n in ((32, 240.0, 2048), (12, 40.0, 300), (8, 30.0, 100), (10, 100.0, 700), (2, 5.0, 20)):
+        got = distance_rows(rows, far, n).tolist()
+        assert got == [P.distance_bucket(i, rows, far) for i in range(n)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_first_tokens_of_a_sequence(dtype):
+    """Requests of one and of two tokens, and the first rows of a longer one, on slots that a longer request
+    has just left: nothing of the request before shows."""
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    runner = runner_for(folder, dtype, max_requests=1)
+    long = random_tokens(vocab, 90, 3)
+    replay(runner, {"long": long}, [{"long": 90}])
+    for n in (1, 2, 5):
+        toks = random_tokens(vocab, n, 100 + n)
+        got = replay(runner, {"s": toks}, [{"s": 1}] * n)["s"]
+        assert_close(got, plain(folder, toks), dtype, f"{n} first tokens")
+
+
+# ------------------------------------------------------------------ the kernels' two paths for experts
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_few_rows_and_many_rows_of_routed_experts_agree_with_the_plain_sum(dtype):
+    from nanoinfer_amd import kernels as K
+    g = torch.Generator().manual_seed(4)
+    T, d, ff, E, top = 12, 48, 24, 7, 3
+    x = torch.randn(T, d, generator=g)
+    up = torch.randn(E * ff, d, generator=g) * 0.3
+    down = torch.randn(d, E * ff, generator=g) * 0.3
+    z = torch.randn(T, E, generator=g)
+    dev = torch.device("cuda")
+    xd, upd, downd = (t.to(dev, dtype).contiguous() for t in (x, up, down))
+    chosen, mix, mix_all = K.route_top(z.to(dev), top, mix_all=True)
+    want = torch.zeros(T, d, dtype=torch.float64)
+    x64, up64, down64 = (t.to(dtype).double() for t in (x, up, down))
+    for t in range(T):
+        idx = torch.topk(z[t], top).indices
+        assert sorted(idx.tolist()) == sorted(chosen[t].tolist())
+        w = torch.softmax(z[t][idx].double(), dim=0)
+        for c, e in enumerate(idx.tolist()):
+            hid = torch.relu(up64[e * ff:(e + 1) * ff] @ x64[t]) ** 2
+            want[t] += w[c] * (down64[:, e * ff:(e + 1) * ff] @ hid)
+    few = K.experts_few(xd, upd, downd, chosen, mix, ff)
+    act = K.experts_act(xd @ upd.t(), mix_all, ff)
+    many = (act.float() @ downd.float().t())
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for name, got in (("few", few), ("many", many)):
+        err = float((got.double().cpu() - want).abs().max() / want.abs().max())
+        assert err < tol, (name, err)
+
+
+# ------------------------------------------------------------------ generation through the entry point
+
+@pytest.mark.parametrize("name", ["mixed", "loop_all"])
+def test_greedy_generation_through_the_engine_is_the_plain_greedy(name):
+    """Requests of unequal length through ``Engine`` (scheduler, chunked prompts, a pool that forces
+    preemptions, runs of recorded decode steps, the sampler's argmax) in float32: the tokens are those
+    that the plain implementation picks, wherever its two largest logits are not a close call."""
+    from nanoinfer_amd.engine.llm import Engine
+    from nanoinfer_amd.engine.scheduler import EngineConfig
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = folder_of(name)
+    config, tensors = P.read_model_folder(folder)
+    vocab, new = config["vocab"], 12
+    prompts = [list(random_tokens(vocab, n, 300 + n)) for n in (3, 41, 17, 1, 66)]
+    eng = Engine(folder, EngineConfig(dtype="float32", block_size=8, num_cache_blocks=24, max_sequences=3,
+                                      prefill_chunk_size=16, max_num_batched_tokens=40), ignore_eos=True)
+    results = eng.generate(prompts, max_new_tokens=new, params=SamplingParams.greedy())
+    assert eng.scheduler.num_preemptions > 0, "the pool was meant to be too small for all"
+    checked = 0
+    for prompt, res in zip(prompts, results):
+        toks = list(prompt)
+        assert len(res.tokens) == new
+        for t in res.tokens:
+            row = P.forward(config, tensors, toks)[-1]
+            top = torch.topk(row, 2).values
+            if float(top[0] - top[1]) > 1e-3 * float(row.abs().max()):
+                assert t == int(row.argmax()), (len(prompt), len(toks))
+                checked += 1
+            toks.append(t)
+    assert checked >= len(prompts) * new * 3 // 4
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages() == eng.runner.cache.num_pages
+
+
+def test_sampling_with_temperature_runs_and_respects_the_seed():
+    from nanoinfer_amd.engine.llm import Engine
+    from nanoinfer_amd.engine.scheduler import EngineConfig
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = folder_of("mixed")
+    prompts = [list(random_tokens(Z.MIXED["vocab"], n, 500 + n)) for n in (9, 20)]
+    outs = []
+    for _ in range(2):
+        eng = Engine(folder, EngineConfig(dtype="bfloat16", block_size=8, num_cache_blocks=64, max_sequences=4), ignore_eos=True)
+        outs.append([r.tokens for r in eng.generate(prompts, max_new_tokens=10,
+                                                    params=SamplingParams(temperature=0.8, top_k=20, top_p=0.9, seed=5))])
+    assert outs[0] == outs[1] and all(len(t) == 10 for t in outs[0])
