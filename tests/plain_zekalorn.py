@@ -156,11 +156,15 @@ def dense_ff(n: torch.Tensor, w: Dict[str, torch.Tensor]) -> torch.Tensor:
     return linear(silu(linear(n, w["gate"])) * linear(n, w["up"]), w["down"])
 
 
-def routed_ff(n: torch.Tensor, w: Dict[str, torch.Tensor], experts: int, top: int) -> torch.Tensor:
+def routed_ff(n: torch.Tensor, w: Dict[str, torch.Tensor], experts: int, top: int, margins: Optional[List] = None) -> torch.Tensor:
     """Every token goes to the ``top`` experts with the largest router logits, weighted by the
-    softmax over those logits alone; an expert is ``Wd relu(Wu n)^2``."""
+    softmax over those logits alone; an expert is ``Wd relu(Wu n)^2``.  ``margins`` collects, per row, by how
+    much the last chosen logit beats the first one left out (how close a call the choice was)."""
     T = n.shape[0]
     z = linear(n, w["router"])
+    if margins is not None and top < experts:
+        ranked = torch.sort(z, dim=-1, descending=True).values
+        margins.append(ranked[:, top - 1] - ranked[:, top])
     out = torch.zeros(T, w["e0.down"].shape[0], dtype=F64)
     for t in range(T):
         chosen = torch.topk(z[t], top).indices
@@ -183,7 +187,8 @@ def sub(tensors: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tensor
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def layer(i: int, x: torch.Tensor, ids: Sequence[int], config: dict, tensors: Dict[str, torch.Tensor]) -> torch.Tensor:
+def layer(i: int, x: torch.Tensor, ids: Sequence[int], config: dict, tensors: Dict[str, torch.Tensor],
+          margins: Optional[List] = None) -> torch.Tensor:
     spec = config["layers"][i]
     eps = config["norm"]["eps"]
     n = rmsnorm(x, tensors[f"l{i}.norm1"], eps)
@@ -200,7 +205,7 @@ def layer(i: int, x: torch.Tensor, ids: Sequence[int], config: dict, tensors: Di
         if mlp["kind"] == "dense":
             y = y + dense_ff(n, ff_w)
         elif mlp["kind"] == "moe":
-            y = y + routed_ff(n, ff_w, mlp["router"]["experts"], mlp["router"]["top"])
+            y = y + routed_ff(n, ff_w, mlp["router"]["experts"], mlp["router"]["top"], margins)
         else:
             raise ValueError(f"feed-forward {mlp['kind']!r}")
     x = x + y
@@ -225,13 +230,15 @@ def layer_runs(config: dict):
     return runs + [(i, None) for i in range(loop["stop"], L)]
 
 
-def forward(config: dict, tensors: Dict[str, torch.Tensor], ids: Sequence[int], streams: Optional[List] = None) -> torch.Tensor:
-    """Logits [T, vocab] of the whole sequence; ``streams`` collects the residual stream after every layer run."""
+def forward(config: dict, tensors: Dict[str, torch.Tensor], ids: Sequence[int], streams: Optional[List] = None,
+            margins: Optional[List] = None) -> torch.Tensor:
+    """Logits [T, vocab] of the whole sequence; ``streams`` collects the residual stream after every layer run,
+    ``margins`` the routers' margins [T] of every routed layer run."""
     x = embed(tensors["embed"], tensors["pos"], config["embedding"]["scale"], ids)
     for i, p in layer_runs(config):
         if p is not None:
             x = x + tensors["loop.step"].to(F64)[p]
-        x = layer(i, x, ids, config, tensors)
+        x = layer(i, x, ids, config, tensors, margins)
         if streams is not None:
             streams.append(x.clone())
     return linear(rmsnorm(x, tensors["final.norm"], config["norm"]["eps"]), tensors["head"])
