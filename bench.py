@@ -137,7 +137,8 @@ class Rig:
         with tempfile.TemporaryDirectory(prefix="nanoinfer-bench-") as folder:
             t0 = time.perf_counter()
             make_random_model(folder, cfg, seed=0, dtype=name)
-            log(f"random model ({cfg['num_hidden_layers']} layers of {cfg['hidden_size']}, {dtype}) written in "
+            log(f"random model ({cfg.get('num_hidden_layers', len(cfg.get('layers', ())))} layers of "
+                f"{cfg.get('hidden_size', cfg.get('width'))}, {dtype}) written in "
                 f"{time.perf_counter() - t0:.1f} s")
             t0 = time.perf_counter()
             self.runner = ModelRunner(folder, dtype=name, page_size=BLOCK_SIZE, max_tokens=pool_tokens,
@@ -152,7 +153,7 @@ class Rig:
         self.torch.cuda.empty_cache()
 
     def prompt(self, n: int):
-        V = self.cfg["vocab_size"]
+        V = self.cfg["vocab_size"] if "vocab_size" in self.cfg else self.cfg["vocab"]
         return [self.rng.randrange(V) for _ in range(n)]
 
     def prefill(self, length: int, chunk: int, recorded: bool = True) -> float:
@@ -379,6 +380,61 @@ def serving(args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------- --workload hybrid
+# A Zekalorn model whose layers have the sizes of the 1B shape's (width 2,048, feed-forwards of 8,192 or sixteen
+# experts of 1,024 of which a token uses four, attention of 32 heads on 8 of size 64, delta-rule layers of 16
+# heads with keys and values of 128), beside the Llama shape of as many layers and the same vocabulary.
+
+def hybrid_config(layers: int, vocab: int, positions: int) -> dict:
+    delta = {"type": "channel_delta", "mixer": {"heads": 16, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4,
+                                                "decay_rank": 64, "gate_rank": 64}}
+    attn = {"type": "attention", "mixer": {"heads": 32, "kv_heads": 8, "dim": 64, "vdim": 64, "scale": 0.125, "bias_max": 4096.0,
+                                           "bias_rows": 64, "q_temp": {"coef": 0.1, "every": 1024}}}
+    dense = {"kind": "dense", "ff": 8192}
+    routed = {"kind": "moe", "expert": {"ff": 1024}, "router": {"experts": 16, "top": 4}}
+    pattern = [(delta, dense), (delta, routed), (delta, dense), (attn, routed)]
+    return {"architecture": "Zekalorn", "vocab": vocab, "width": 2048, "max_positions": positions,
+            "embedding": {"scale": 45.25}, "norm": {"eps": 1e-5}, "token_side": {"dim": 64},
+            "layers": [dict(pattern[i % 4][0], mlp=pattern[i % 4][1]) for i in range(layers)]}
+
+
+def hybrid(args) -> int:
+    """``--workload hybrid``: prefill of one prompt and decode steps of the Zekalorn shape above and of the Llama
+    shape of equal depth, one JSON line with both."""
+    import torch
+    torch.cuda.set_device(0)
+    layers = args.layers or 8
+    prompt, batch = args.prompt_len, args.batch
+    out = {"metric": "hybrid_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "higher_is_better": True, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
+           "config": {"layers": layers, "prompt_len": prompt, "global_batch": batch, "width": 2048, "vocab": 128256}}
+    shapes = {"zekalorn": hybrid_config(layers, 128256, prompt + 2048),
+              "llama": dict(LLAMA_1B, num_hidden_layers=layers, max_position_embeddings=prompt + 2048)}
+    for name, cfg in shapes.items():
+        if args.only and name != args.only:
+            continue
+        rig = Rig(cfg, args.dtype, max(batch, 1) * (prompt + 2048), max(batch, 4), args.decode_run)
+        rec = {}
+        if args.phase in ("all", "prefill"):
+            sec = rig.prefill(prompt, prompt)
+            rec["prefill_tok_s"], rec["prefill_ms"] = round(prompt / sec, 1), round(sec * 1e3, 3)
+            sec = rig.prefill(prompt, 512)
+            rec["prefill_512_tok_s"] = round(prompt / sec, 1)
+        if args.phase in ("all", "decode"):
+            for b in sorted({1, batch}):
+                step_s, ctx = rig.decode(b, prompt, args.steps, args.warmup)
+                rec[f"decode_b{b}_tok_s"], rec[f"decode_b{b}_step_ms"] = round(b / step_s, 1), round(step_s * 1e3, 4)
+        rec["weights_gb"] = round(rig.runner.memory_report()["weights"] / 1e9, 3)
+        out[name] = rec
+        log(f"{name}: {rec}")
+        rig.close()
+    if "zekalorn" in out and f"decode_b{batch}_tok_s" in out["zekalorn"]:
+        out["value"] = out["zekalorn"][f"decode_b{batch}_tok_s"]
+        out["ms_per_step"] = out["zekalorn"][f"decode_b{batch}_step_ms"]
+    print(json.dumps(out))
+    return 0
+
+
 def serving_brief(full: dict) -> dict:
     """The figures of a serving result that go onto the default line, flat."""
     return {"value": full["value"], "total_ms": full["total_ms"], "requests": full["config"]["requests"],
@@ -410,9 +466,11 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the further points")
     ap.add_argument("--no-further", action="store_true",
                     help="skip the points beyond the contract's: contexts of 8k and 32k, float32, the 3B shape")
-    ap.add_argument("--workload", default="steps", choices=["steps", "serving"],
+    ap.add_argument("--only", default=None, choices=["zekalorn", "llama"], help="hybrid: measure one of the two models")
+    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid"],
                     help="steps: the decode step and prefill of the result line's contract (default); "
-                         "serving: concurrent requests through the engine's scheduler, a line of its own")
+                         "serving: concurrent requests through the engine's scheduler, a line of its own; "
+                         "hybrid: prefill and decode of a Zekalorn model at the 1B shape's layer sizes beside the Llama shape")
     ap.add_argument("--requests", type=int, default=64, help="serving: concurrent requests")
     ap.add_argument("--new-tokens", type=int, default=256, help="serving: tokens generated per request")
     ap.add_argument("--min-prompt", type=int, default=128, help="serving: shortest prompt")
@@ -433,6 +491,8 @@ def main() -> int:
         return 2
     if args.workload == "serving":
         return serving(args)
+    if args.workload == "hybrid":
+        return hybrid(args)
     args.prefill_chunk = args.prefill_chunk or PREFILL_CHUNK
 
     import torch

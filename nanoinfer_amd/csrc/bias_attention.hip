@@ -49,14 +49,17 @@ __global__ void __launch_bounds__(WAVES * WAVE)
 bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
                       const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
-                      int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk) {
+                      int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk, int n_runs,
+                      float* __restrict__ partial) {
     extern __shared__ float lds[];
     const int dkp = dk + 1;                       // a lane reads its key's row: odd strides spread the banks
     float* Qs = lds;                              // [ROWS][dk]
     float* Ks = Qs + ROWS * dk;                   // [KEYS][dkp]
     float* Vs = Ks + KEYS * dkp;                  // [KEYS][dv]
     float* Ps = Vs + KEYS * dv;                   // [WAVES][ROWS_PER_WAVE][KEYS]
-    const int tile = blockIdx.x, g = blockIdx.y, chunk = blockIdx.z;
+    // with n_runs > 1 the keys of a tile are cut into runs, one workgroup each, whose (maximum, sum, weighted
+    // sum) a second kernel merges: a single token over thousands of keys then fills the chip
+    const int tile = blockIdx.x / n_runs, run = blockIdx.x % n_runs, g = blockIdx.y, chunk = blockIdx.z;
     // the first position is read from the step's positions, not from the tile: a recorded decode step is replayed
     // with new positions and the tiles it was recorded with
     const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2];
@@ -91,13 +94,15 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
         for (int cc = 0; cc < MAX_VCHUNKS; ++cc) acc[rr][cc] = 0.f;
     }
     const int last_pos = first_pos + n_tok - 1;
+    const int span = ((last_pos + n_runs) / n_runs + KEYS - 1) / KEYS * KEYS;      // keys of a run: whole tiles of 64
+    const int k_begin = run * span, k_last = std::min(last_pos, k_begin + span - 1);
     const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
-    for (int k0 = 0; k0 <= last_pos; k0 += KEYS) {
+    for (int k0 = k_begin; k0 <= k_last; k0 += KEYS) {
         __syncthreads();                          // the tile before this one has been used by everyone
         for (int i = tid; i < KEYS * dk; i += blockDim.x) {
             const int j = i / dk, c = i % dk, key = k0 + j;
             float v = 0.f;
-            if (key <= last_pos) {
+            if (key <= k_last) {
                 const int page = table[key / page_size];
                 if (page >= 0) v = ld(kpool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * dk + c);
             }
@@ -106,7 +111,7 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
         for (int i = tid; i < KEYS * dv; i += blockDim.x) {
             const int j = i / dv, c = i % dv, key = k0 + j;
             float v = 0.f;
-            if (key <= last_pos) {
+            if (key <= k_last) {
                 const int page = table[key / page_size];
                 if (page >= 0) v = ld(vpool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * dv + c);
             }
@@ -132,7 +137,7 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
             alpha[rr] = 1.f;
             if (!valid[rr]) { prow[rr * KEYS + lane] = 0.f; continue; }          // the same for the whole wavefront
             if (k0 > pos[rr]) { prow[rr * KEYS + lane] = 0.f; continue; }        // the same for the whole wavefront
-            const bool seen = key <= pos[rr];
+            const bool seen = key <= pos[rr] && key <= k_last;
             float sc = -INFINITY;
             if (seen) {
                 const int back = std::min(pos[rr] - key, distances - 1);
@@ -168,6 +173,16 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
     for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
         if (!valid[rr]) continue;
         const int r = wave * ROWS_PER_WAVE + rr;
+        if (partial) {
+            float* prow = partial + ((static_cast<size_t>(first_row + r / heads_here) * H + head[rr]) * n_runs + run) * (dv + 2);
+            if (lane == 0) { prow[0] = m[rr]; prow[1] = l[rr]; }
+#pragma unroll
+            for (int cc = 0; cc < MAX_VCHUNKS; ++cc) {
+                const int c = lane + cc * WAVE;
+                if (c < dv) prow[2 + c] = acc[rr][cc];
+            }
+            continue;
+        }
         T* orow = out + static_cast<size_t>(first_row + r / heads_here) * (H * dv) + head[rr] * dv;
         const float inv = 1.0f / l[rr];
 #pragma unroll
@@ -175,6 +190,26 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
             const int c = lane + cc * WAVE;
             if (c < dv) st(orow + c, acc[rr][cc] * inv);
         }
+    }
+}
+
+// out[row, :] = sum_r acc_r e^(m_r - M) / sum_r l_r e^(m_r - M) over the runs of a row (an empty run has l = 0)
+template <typename T>
+__global__ void merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv) {
+    const size_t row = blockIdx.x;
+    const float* p = partial + row * n_runs * (dv + 2);
+    float M = -INFINITY;
+    for (int r = 0; r < n_runs; ++r) M = fmaxf(M, p[r * (dv + 2)]);
+    float L = 0.f;
+    for (int r = 0; r < n_runs; ++r) {
+        const float l = p[r * (dv + 2) + 1];
+        if (l > 0.f) L += l * expf(p[r * (dv + 2)] - M);
+    }
+    for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+        float a = 0.f;
+        for (int r = 0; r < n_runs; ++r)
+            if (p[r * (dv + 2) + 1] > 0.f) a += p[r * (dv + 2) + 2 + c] * expf(p[r * (dv + 2)] - M);
+        st(out + row * dv + c, a / L);
     }
 }
 
@@ -195,14 +230,16 @@ NI_EXPORT int ni_bias_attention_rows() { return ROWS; }
 NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
                                 int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias, int distances, void* out,
                                 int H, int G, int dk, int dv, int page_size, float scale, float temp_coef, int temp_every,
-                                int heads_per_chunk, int dtype, hipStream_t stream) {
+                                int heads_per_chunk, int n_runs, void* partial, int n_rows, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
     if (dv > MAX_VCHUNKS * WAVE || H % G || heads_per_chunk < 1 || heads_per_chunk > ROWS) return -1;
     const int group = H / G;
     const size_t lds = (static_cast<size_t>(ROWS) * dk + static_cast<size_t>(KEYS) * (dk + 1) + static_cast<size_t>(KEYS) * dv +
                         WAVES * ROWS_PER_WAVE * KEYS) * sizeof(float);
     if (lds > 160 * 1024) return -2;
-    dim3 grid(n_tiles, G, (group + heads_per_chunk - 1) / heads_per_chunk);
+    if (n_runs < 1 || (n_runs > 1 && !partial)) return -1;
+    if (n_runs == 1) partial = nullptr;
+    dim3 grid(n_tiles * n_runs, G, (group + heads_per_chunk - 1) / heads_per_chunk);
     hipError_t err = hipSuccess;
     if (dtype == 0) {
         static size_t allowed = 48 * 1024;
@@ -212,7 +249,8 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk);
+            temp_every, heads_per_chunk, n_runs, (float*)partial);
+        if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv);
     } else {
         static size_t allowed = 48 * 1024;
         if (lds > allowed && (allowed = lds))
@@ -221,7 +259,8 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk);
+            temp_every, heads_per_chunk, n_runs, (float*)partial);
+        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv);
     }
     return NI_LAUNCH_RESULT();
 }

@@ -36,6 +36,20 @@ __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log
 // conv float32 [C, taps] with C = 2*G*dk + H*dv (the filters of q, k, v stacked).
 // state float32 [slots, state_stride]; the convolutions' inputs lie at conv_off as [taps - 1, C].
 // prep float32 [T, prep_cols]: q | k | v | beta [H] | g [H*dk] | gate [H*dv].
+// One workgroup a (token, unit): units 0 .. 2G-1 are the heads of q and of k (convolution, silu, unit norm),
+// units 2G .. 2G+H-1 the heads of v with that head's beta, decay and gate.
+__device__ __forceinline__ float conv_at(const float* __restrict__ proj, const float* __restrict__ hist,
+                                         const float* __restrict__ conv, int t, int i, int c, int C, int taps, int proj_cols) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j;
+        const float x = (i - back >= 0) ? proj[static_cast<size_t>(t - back) * proj_cols + c]
+                                        : hist[static_cast<size_t>(taps - 1 + i - back) * C + c];
+        acc += conv[static_cast<size_t>(c) * taps + j] * x;
+    }
+    return acc;
+}
+
 __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float* __restrict__ low,
                                      const float* __restrict__ conv, const float* __restrict__ a_log,
                                      const float* __restrict__ dt_bias, const float* __restrict__ state,
@@ -43,44 +57,42 @@ __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float
                                      const int32_t* __restrict__ state_slot, float* __restrict__ prep,
                                      int G, int H, int dk, int dv, int taps, int proj_cols, size_t state_stride,
                                      size_t conv_off) {
-    extern __shared__ float qk[];              // q then k after convolution and silu: 2 * G * dk
-    const int t = blockIdx.x;
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, unit = blockIdx.y;
     const int s = seq_of_token[t];
     const int i = t - q_start[s];              // place of the token in its portion
     const int QK = 2 * G * dk, C = QK + H * dv;
     const int prep_cols = C + H + H * dk + H * dv;
     const float* hist = state + static_cast<size_t>(state_slot[s]) * state_stride + conv_off;
     float* out = prep + static_cast<size_t>(t) * prep_cols;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-        float acc = 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int back = taps - 1 - j;
-            const float x = (i - back >= 0) ? proj[static_cast<size_t>(t - back) * proj_cols + c]
-                                            : hist[static_cast<size_t>(taps - 1 + i - back) * C + c];
-            acc += conv[static_cast<size_t>(c) * taps + j] * x;
+    if (unit < 2 * G) {
+        // a head of q or of k: every thread keeps its channels (dk <= 256 = threads)
+        const int c = unit * dk + threadIdx.x;
+        float y = 0.f;
+        if (threadIdx.x < dk) {
+            const float z = conv_at(proj, hist, conv, t, i, c, C, taps, proj_cols);
+            y = z * (1.0f / (1.0f + expf(-z)));
         }
-        const float y = silu_f(acc);
-        if (c < QK) qk[c] = y; else out[c] = y;
+        const float ss = block_sum(y * y, scratch);
+        const float inv = (1.0f / sqrtf(ss + 1e-6f)) * (unit < G ? 1.0f / sqrtf(static_cast<float>(dk)) : 1.0f);
+        if (threadIdx.x < dk) out[c] = y * inv;
+        return;
     }
-    // beta, decay, gate
+    const int h = unit - 2 * G;
     const float* prow = proj + static_cast<size_t>(t) * proj_cols;
     const float* lrow = low + static_cast<size_t>(t) * (H * dk + H * dv);
-    for (int c = threadIdx.x; c < H; c += blockDim.x) out[C + c] = sigmoid_f(prow[C + c]);
-    for (int c = threadIdx.x; c < H * dk; c += blockDim.x)
-        out[C + H + c] = expf(-expf(a_log[c / dk]) * softplus_f(lrow[c] + dt_bias[c]));
-    for (int c = threadIdx.x; c < H * dv; c += blockDim.x) out[C + H + H * dk + c] = sigmoid_f(lrow[H * dk + c]);
-    __syncthreads();
-    // unit vectors per head of q and of k; q also times dk^(-1/2)
-    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
-    const float qscale = 1.0f / sqrtf(static_cast<float>(dk));
-    for (int head = wave; head < 2 * G; head += waves) {
-        const float* v = qk + head * dk;
-        float ss = 0.f;
-        for (int c = lane; c < dk; c += WAVE) ss += v[c] * v[c];
-        ss = wave_sum(ss);
-        const float inv = (1.0f / sqrtf(ss + 1e-6f)) * (head < G ? qscale : 1.0f);
-        for (int c = lane; c < dk; c += WAVE) out[head * dk + c] = v[c] * inv;
+    for (int j = threadIdx.x; j < dv; j += blockDim.x) {
+        const int c = QK + h * dv + j;
+        const float z = conv_at(proj, hist, conv, t, i, c, C, taps, proj_cols);
+        out[c] = z * (1.0f / (1.0f + expf(-z)));
+        out[C + H + H * dk + h * dv + j] = 1.0f / (1.0f + expf(-lrow[H * dk + h * dv + j]));
     }
+    const float rate = expf(a_log[h]);
+    for (int j = threadIdx.x; j < dk; j += blockDim.x) {
+        const float z = lrow[h * dk + j] + dt_bias[h * dk + j];
+        out[C + H + h * dk + j] = expf(-rate * (z > 20.f ? z : log1pf(expf(z))));
+    }
+    if (threadIdx.x == 0) out[C + h] = 1.0f / (1.0f + expf(-prow[C + h]));
 }
 
 __global__ void conv_state_update_kernel(const float* __restrict__ proj, float* __restrict__ state,
@@ -100,68 +112,95 @@ __global__ void conv_state_update_kernel(const float* __restrict__ proj, float* 
     }
 }
 
-// One workgroup: COLS = 256 / PARTS value channels of one head of one sequence.
+// One workgroup: COLS = 256 / PARTS value channels of one head of one sequence.  The operands of CHUNK tokens at a
+// time (q, k and g of the head, the workgroup's channels of v, beta) are brought into LDS by all threads together
+// while the chunk before is worked through: the recurrence itself then waits for no load from memory, which at one
+// token after the other would cost a round trip each.
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(const float* __restrict__ prep, float* __restrict__ state, const int32_t* __restrict__ q_start,
                   const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, float* __restrict__ o,
                   int G, int H, int dv, size_t state_stride) {
     constexpr int DK = KPT * PARTS, COLS = 256 / PARTS;
+    constexpr int CHUNK = DK <= 128 ? 16 : 8;
+    constexpr int ROW = 3 * DK + COLS + 1;                    // q | k | g | v of the workgroup's channels | beta
+    constexpr int LOADS = (CHUNK * ROW + 255) / 256;
+    __shared__ float buf[2][CHUNK * ROW];
     const int s = blockIdx.x, h = blockIdx.y;
     const int part = threadIdx.x % PARTS;
-    const int col = blockIdx.z * COLS + threadIdx.x / PARTS;
+    const int col0 = blockIdx.z * COLS;
+    const int lcol = threadIdx.x / PARTS, col = col0 + lcol;
     const bool live = col < dv;
     const int g = h / (H / G);
     const int QK = 2 * G * DK, C = QK + H * dv;
     const int prep_cols = C + H + H * DK + H * dv;
-    const int n = q_len[s];
-    const float* row = prep + static_cast<size_t>(q_start[s]) * prep_cols;
+    const int n = q_len[s], first = q_start[s];
+    const float* rows = prep + static_cast<size_t>(first) * prep_cols;
     float* S_mem = state + static_cast<size_t>(state_slot[s]) * state_stride +
                    (static_cast<size_t>(h) * dv + (live ? col : 0)) * DK + part * KPT;
     float S[KPT];
 #pragma unroll
     for (int i = 0; i < KPT; ++i) S[i] = live ? S_mem[i] : 0.f;
-    const int q_at = g * DK + part * KPT, k_at = G * DK + g * DK + part * KPT;
-    const int v_at = QK + h * dv + (live ? col : 0), b_at = C + h, g_at = C + H + h * DK + part * KPT;
-    float q[KPT], k[KPT], dec[KPT], v, beta;
+
+    float stage[LOADS];
+    auto fetch = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) { q[i] = row[q_at + i]; k[i] = row[k_at + i]; dec[i] = row[g_at + i]; }
-    v = row[v_at];
-    beta = row[b_at];
-    for (int t = 0; t < n; ++t) {
-        // the next token's operands are asked for before this token's arithmetic
-        float qn[KPT], kn[KPT], dn[KPT], vn = 0.f, bn = 0.f;
-        const bool more = t + 1 < n;
-        const float* next = row + prep_cols;
-#pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-            qn[i] = more ? next[q_at + i] : 0.f;
-            kn[i] = more ? next[k_at + i] : 0.f;
-            dn[i] = more ? next[g_at + i] : 0.f;
+        for (int j = 0; j < LOADS; ++j) {
+            const int e = threadIdx.x + j * 256;
+            const int tok = e / ROW, r = e % ROW;
+            float v = 0.f;
+            if (e < CHUNK * ROW && t0 + tok < n) {
+                const float* row = rows + static_cast<size_t>(t0 + tok) * prep_cols;
+                if (r < DK) v = row[g * DK + r];
+                else if (r < 2 * DK) v = row[G * DK + g * DK + (r - DK)];
+                else if (r < 3 * DK) v = row[C + H + h * DK + (r - 2 * DK)];
+                else if (r < 3 * DK + COLS) { if (col0 + (r - 3 * DK) < dv) v = row[QK + h * dv + col0 + (r - 3 * DK)]; }
+                else v = row[C + h];
+            }
+            stage[j] = v;
         }
-        if (more) { vn = next[v_at]; bn = next[b_at]; }
-        float a = 0.f, b = 0.f, kq = 0.f;
+    };
+    auto put = [&](float* dst) {
 #pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-            S[i] *= dec[i];
-            a += S[i] * k[i];
-            b += S[i] * q[i];
-            kq += k[i] * q[i];
+        for (int j = 0; j < LOADS; ++j) {
+            const int e = threadIdx.x + j * 256;
+            if (e < CHUNK * ROW) dst[e] = stage[j];
         }
+    };
+    fetch(0);
+    put(buf[0]);
+    __syncthreads();
+    int which = 0;
+    for (int t0 = 0; t0 < n; t0 += CHUNK) {
+        const bool more = t0 + CHUNK < n;
+        if (more) fetch(t0 + CHUNK);
+        const float* cur = buf[which];
+        const int count = min(CHUNK, n - t0);
+        for (int tt = 0; tt < count; ++tt) {
+            const float* r = cur + tt * ROW;
+            float a = 0.f, b = 0.f, kq = 0.f, k[KPT];
 #pragma unroll
-        for (int off = 1; off < PARTS; off <<= 1) {
-            a += __shfl_xor(a, off, WAVE);
-            b += __shfl_xor(b, off, WAVE);
-            kq += __shfl_xor(kq, off, WAVE);
+            for (int i = 0; i < KPT; ++i) {
+                const float q = r[part * KPT + i];
+                k[i] = r[DK + part * KPT + i];
+                S[i] *= r[2 * DK + part * KPT + i];
+                a += S[i] * k[i];
+                b += S[i] * q;
+                kq += k[i] * q;
+            }
+#pragma unroll
+            for (int off = 1; off < PARTS; off <<= 1) {
+                a += __shfl_xor(a, off, WAVE);
+                b += __shfl_xor(b, off, WAVE);
+                kq += __shfl_xor(kq, off, WAVE);
+            }
+            const float u = r[3 * DK + COLS] * (r[3 * DK + lcol] - a);
+#pragma unroll
+            for (int i = 0; i < KPT; ++i) S[i] += k[i] * u;
+            if (live && part == 0) o[(static_cast<size_t>(first) + t0 + tt) * (H * dv) + h * dv + col] = b + u * kq;
         }
-        const float u = beta * (v - a);
-#pragma unroll
-        for (int i = 0; i < KPT; ++i) S[i] += k[i] * u;
-        if (live && part == 0) o[(static_cast<size_t>(q_start[s]) + t) * (H * dv) + h * dv + col] = b + u * kq;
-#pragma unroll
-        for (int i = 0; i < KPT; ++i) { q[i] = qn[i]; k[i] = kn[i]; dec[i] = dn[i]; }
-        v = vn;
-        beta = bn;
-        row = next;
+        if (more) put(buf[which ^ 1]);
+        __syncthreads();
+        which ^= 1;
     }
     if (live) {
 #pragma unroll
@@ -195,9 +234,8 @@ NI_EXPORT int ni_delta_prepare(const void* proj, const void* low, const void* co
     if (T <= 0) return 0;
     if (dk != KPT * PARTS) return -1;
     const int C = 2 * G * dk + H * dv;
-    const size_t lds = static_cast<size_t>(2 * G * dk) * sizeof(float);
-    if (lds > 64 * 1024) return -2;
-    delta_prepare_kernel<<<T, 256, lds, stream>>>((const float*)proj, (const float*)low, (const float*)conv,
+    if (dk > 256) return -2;
+    delta_prepare_kernel<<<dim3(T, 2 * G + H), 256, 0, stream>>>((const float*)proj, (const float*)low, (const float*)conv,
                                                   (const float*)a_log, (const float*)dt_bias, (const float*)state,
                                                   (const int32_t*)seq_of_token, (const int32_t*)q_start,
                                                   (const int32_t*)state_slot, (float*)prep, G, H, dk, dv, taps, proj_cols,

@@ -9,6 +9,9 @@
 #include <algorithm>
 
 static inline unsigned blocks_of(size_t n, unsigned per) { return static_cast<unsigned>((n + per - 1) / per); }
+static inline bool aligned16(const void* a, const void* b) {
+    return (reinterpret_cast<uintptr_t>(a) % 16 == 0) && (reinterpret_cast<uintptr_t>(b) % 16 == 0);
+}
 
 __device__ __forceinline__ float gelu_tanh_f(float z) {
     // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
@@ -229,7 +232,7 @@ NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int
 //   out[t, r] = sum_k mix[t, k] * W_down[r, chosen[t, k] * ff : +ff] . hid[t * top + k, :]
 template <typename T>
 __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restrict__ w_up, const int32_t* __restrict__ chosen,
-                                      float* __restrict__ hid, int d, int ff, int top, int rows_per_block) {
+                                      float* __restrict__ hid, int d, int ff, int top, int rows_per_block, bool vec) {
     const int pair = blockIdx.x;                 // t * top + k
     const int t = pair / top;
     const int e = chosen[pair];
@@ -239,7 +242,17 @@ __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restri
     for (int i = first + wave; i < first + rows_per_block && i < ff; i += waves) {
         const T* wr = w_up + (static_cast<size_t>(e) * ff + i) * d;
         float s = 0.f;
-        for (int c = lane; c < d; c += WAVE) s += ld(wr + c) * ld(xr + c);
+        if (vec) {          // eight elements a lane and load: a wavefront takes 512 neighbouring elements at once
+            for (int c = lane * 8; c < d; c += WAVE * 8) {
+                float wv[8], xv[8];
+                VecIO<T, 8>::load(wr + c, wv);
+                VecIO<T, 8>::load(xr + c, xv);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) s += wv[j] * xv[j];
+            }
+        } else {
+            for (int c = lane; c < d; c += WAVE) s += ld(wr + c) * ld(xr + c);
+        }
         s = wave_sum(s);
         if (lane == 0) {
             const float u = fmaxf(s, 0.f);
@@ -251,7 +264,7 @@ __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restri
 template <typename T>
 __global__ void experts_down_few_kernel(const float* __restrict__ hid, const T* __restrict__ w_down,
                                         const int32_t* __restrict__ chosen, const float* __restrict__ mix,
-                                        float* __restrict__ out, int d, int ff, int E, int top, int rows_per_block) {
+                                        float* __restrict__ out, int d, int ff, int E, int top, int rows_per_block, bool vec) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
     const int first = blockIdx.y * rows_per_block;
@@ -263,7 +276,17 @@ __global__ void experts_down_few_kernel(const float* __restrict__ hid, const T* 
             const T* wr = w_down + static_cast<size_t>(r) * row_stride + static_cast<size_t>(e) * ff;
             const float* hr = hid + (static_cast<size_t>(t) * top + k) * ff;
             float s = 0.f;
-            for (int c = lane; c < ff; c += WAVE) s += ld(wr + c) * hr[c];
+            if (vec) {
+                for (int c = lane * 8; c < ff; c += WAVE * 8) {
+                    float wv[8], hv[8];
+                    VecIO<T, 8>::load(wr + c, wv);
+                    VecIO<float, 8>::load(hr + c, hv);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) s += wv[j] * hv[j];
+                }
+            } else {
+                for (int c = lane; c < ff; c += WAVE) s += ld(wr + c) * hr[c];
+            }
             total += mix[t * top + k] * wave_sum(s);
         }
         if (lane == 0) out[static_cast<size_t>(t) * d + r] = total;
@@ -275,16 +298,19 @@ NI_EXPORT int ni_experts_few(const void* x, const void* w_up, const void* w_down
     if (T <= 0) return 0;
     const int rows = 16;
     dim3 g1(T * top, (ff + rows - 1) / rows), g2(T, (d + rows - 1) / rows);
+    // rows of whole 16-byte (bfloat16) or 32-byte (float32) pieces that start on such a piece are read in pieces
+    const bool vec_up = d % 8 == 0 && aligned16(x, w_up);
+    const bool vec_down = ff % 8 == 0 && aligned16(w_down, hid);
     if (dtype == 0) {
         experts_up_few_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)w_up, (const int32_t*)chosen,
-                                                             (float*)hid, d, ff, top, rows);
+                                                             (float*)hid, d, ff, top, rows, vec_up);
         experts_down_few_kernel<float><<<g2, 256, 0, stream>>>((const float*)hid, (const float*)w_down, (const int32_t*)chosen,
-                                                               (const float*)mix, (float*)out, d, ff, E, top, rows);
+                                                               (const float*)mix, (float*)out, d, ff, E, top, rows, vec_down);
     } else {
         experts_up_few_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w_up, (const int32_t*)chosen,
-                                                              (float*)hid, d, ff, top, rows);
+                                                              (float*)hid, d, ff, top, rows, vec_up);
         experts_down_few_kernel<bf16_t><<<g2, 256, 0, stream>>>((const float*)hid, (const bf16_t*)w_down, (const int32_t*)chosen,
-                                                                (const float*)mix, (float*)out, d, ff, E, top, rows);
+                                                                (const float*)mix, (float*)out, d, ff, E, top, rows, vec_down);
     }
     return NI_LAUNCH_RESULT();
 }

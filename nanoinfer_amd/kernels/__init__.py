@@ -1185,5 +1185,5 @@ torch.backends.cudnn.allow_tf32 = False
 
 # sums onto the residual stream, routed experts, the gated delta rule, attention with a bias by distance
 from .stream import (EXPERTS_FEW_ROWS, add_rmsnormed, add_vector, bias_attention, bias_attention_lib,  # noqa: E402,F401
-                     bias_attention_rows, delta_rule, delta_rule_lib, embed_scaled, experts_act, experts_few,
+                     bias_attention_rows, bias_attention_runs, delta_rule, delta_rule_lib, embed_scaled, experts_act, experts_few,
                      gated_side, kv_store, route_top, stream_add, stream_lib)

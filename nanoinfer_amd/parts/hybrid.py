@@ -210,8 +210,11 @@ class BiasAttention(Part):
         if tiles is None:
             raise K.KernelError("this step was recorded without the tiles of its tokens")
         out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
+        chunks = -(-(self.H // self.G) // self.heads_per_chunk)
+        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, ctx.max_context)
+        ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
         K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H, self.scale,
-                         self.temp_coef, self.temp_every, self.heads_per_chunk)
+                         self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws)
         return K.linear(out, self.w_o, out_dtype=torch.float32)
 
 

@@ -247,16 +247,20 @@ def _far_sighted(tensors):
         tensors[k] = (tensors[k].float() * 2.0).to(torch.bfloat16)
 
 
+@pytest.mark.parametrize("run_keys", [256, 64])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_far_keys_and_edges_of_pages_and_key_runs(dtype):
+def test_far_keys_and_edges_of_pages_and_key_runs(dtype, run_keys, monkeypatch):
     """A head whose bias prefers the farthest keys: prompts that end, portions that start and
     single tokens that fall just before, on and just behind the edges of pages (8) and of the kernel's runs of
     64 keys, over a few hundred keys."""
+    import nanoinfer_amd.kernels.stream as stream
+    monkeypatch.setattr(stream, "RUN_KEYS", run_keys)      # 64: steps of few tokens cut their keys into runs that are merged
     name = "attention_only"
     folder = folder_of(name, edit=_far_sighted)
     toks = random_tokens(Z.ALL[name]["vocab"], 330, 9)
     want = plain(folder, toks)
     runner = runner_for(folder, dtype)
+    assert stream.bias_attention_runs(1, 2, 1, 300) == (1 if run_keys == 256 else 4)
     for first in (63, 64, 65, 127, 128, 129, 7, 8, 9, 255, 257):
         rest = len(toks) - first
         steps = [{"k": first}] + [{"k": 1}] * 3 + [{"k": c} for c in cuts(rest - 3, [62, 2, 1, 64, 3])]
