@@ -44,13 +44,65 @@ __global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k
     }
 }
 
+// 64 rows of a pool (keys or values of one kv head) from their pages into LDS as float32, row stride `stride`.
+// With `pieces` (rows of whole 16-byte pieces, 16-byte aligned) a thread asks for four pieces before it stores
+// the first: the loads of a tile are then in flight together instead of one round trip after the other.
+template <typename T>
+__device__ __forceinline__ void stage_rows(const T* __restrict__ pool, float* __restrict__ dst, int stride, int size,
+                                           const int32_t* __restrict__ table, int page_size, int G, int g, int k0,
+                                           int k_last, bool pieces) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int tid = threadIdx.x, threads = blockDim.x;
+    if (pieces) {
+        const int per_row = size / VEC, total = KEYS * per_row;
+        for (int base = 0; base < total; base += 4 * threads) {
+            RawRow<T, VEC> raw[4];
+            bool have[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * threads + tid;
+                have[u] = false;
+                if (idx < total) {
+                    const int j = idx / per_row, pc = idx % per_row, key = k0 + j;
+                    if (key <= k_last) {
+                        const int page = table[key / page_size];
+                        if (page >= 0) {
+                            raw[u].load(pool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * size + pc * VEC);
+                            have[u] = true;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * threads + tid;
+                if (idx < total) {
+                    float* d = dst + (idx / per_row) * stride + (idx % per_row) * VEC;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) d[e] = have[u] ? raw[u].get(e) : 0.f;
+                }
+            }
+        }
+        return;
+    }
+    for (int i = tid; i < KEYS * size; i += threads) {
+        const int j = i / size, c = i % size, key = k0 + j;
+        float v = 0.f;
+        if (key <= k_last) {
+            const int page = table[key / page_size];
+            if (page >= 0) v = ld(pool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * size + c);
+        }
+        dst[j * stride + c] = v;
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(WAVES * WAVE)
 bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
                       const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
                       int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk, int n_runs,
-                      float* __restrict__ partial) {
+                      float* __restrict__ partial, bool k_pieces, bool v_pieces) {
     extern __shared__ float lds[];
     const int dkp = dk + 1;                       // a lane reads its key's row: odd strides spread the banks
     float* Qs = lds;                              // [ROWS][dk]
@@ -99,24 +151,8 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
     const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
     for (int k0 = k_begin; k0 <= k_last; k0 += KEYS) {
         __syncthreads();                          // the tile before this one has been used by everyone
-        for (int i = tid; i < KEYS * dk; i += blockDim.x) {
-            const int j = i / dk, c = i % dk, key = k0 + j;
-            float v = 0.f;
-            if (key <= k_last) {
-                const int page = table[key / page_size];
-                if (page >= 0) v = ld(kpool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * dk + c);
-            }
-            Ks[j * dkp + c] = v;
-        }
-        for (int i = tid; i < KEYS * dv; i += blockDim.x) {
-            const int j = i / dv, c = i % dv, key = k0 + j;
-            float v = 0.f;
-            if (key <= k_last) {
-                const int page = table[key / page_size];
-                if (page >= 0) v = ld(vpool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * dv + c);
-            }
-            Vs[i] = v;
-        }
+        stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, k_last, k_pieces);
+        stage_rows<T>(vpool, Vs, dv, dv, table, page_size, G, g, k0, k_last, v_pieces);
         __syncthreads();
         // scores of this lane's key for the wavefront's rows
         float s[ROWS_PER_WAVE];
@@ -230,14 +266,17 @@ NI_EXPORT int ni_bias_attention_rows() { return ROWS; }
 NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
                                 int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias, int distances, void* out,
                                 int H, int G, int dk, int dv, int page_size, float scale, float temp_coef, int temp_every,
-                                int heads_per_chunk, int n_runs, void* partial, int n_rows, int dtype, hipStream_t stream) {
+                                int heads_per_chunk, int n_runs, void* partial, int n_rows, int waves, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
     if (dv > MAX_VCHUNKS * WAVE || H % G || heads_per_chunk < 1 || heads_per_chunk > ROWS) return -1;
     const int group = H / G;
     const size_t lds = (static_cast<size_t>(ROWS) * dk + static_cast<size_t>(KEYS) * (dk + 1) + static_cast<size_t>(KEYS) * dv +
                         WAVES * ROWS_PER_WAVE * KEYS) * sizeof(float);
     if (lds > 160 * 1024) return -2;
-    if (n_runs < 1 || (n_runs > 1 && !partial)) return -1;
+    if (n_runs < 1 || (n_runs > 1 && !partial) || waves < 1 || waves > WAVES) return -1;
+    const int vec = dtype == 0 ? 4 : 8;
+    const bool k_pieces = dk % vec == 0 && reinterpret_cast<uintptr_t>(kpool) % 16 == 0;
+    const bool v_pieces = dv % vec == 0 && reinterpret_cast<uintptr_t>(vpool) % 16 == 0;
     if (n_runs == 1) partial = nullptr;
     dim3 grid(n_tiles * n_runs, G, (group + heads_per_chunk - 1) / heads_per_chunk);
     hipError_t err = hipSuccess;
@@ -246,20 +285,20 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         if (lds > allowed && (allowed = lds))
             err = hipFuncSetAttribute((const void*)bias_attention_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return (int)err;
-        bias_attention_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
+        bias_attention_kernel<float><<<grid, waves * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces);
         if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv);
     } else {
         static size_t allowed = 48 * 1024;
         if (lds > allowed && (allowed = lds))
             err = hipFuncSetAttribute((const void*)bias_attention_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return (int)err;
-        bias_attention_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
+        bias_attention_kernel<bf16_t><<<grid, waves * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces);
         if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv);
     }
     return NI_LAUNCH_RESULT();

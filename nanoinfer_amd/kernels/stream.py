@@ -195,16 +195,16 @@ def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log:
 
 # ------------------------------------------------------------------ attention with a bias by distance
 
-RUN_KEYS = 256      # a run of keys is at least this long
+RUN_KEYS = 128      # a run of keys is at least this long
 
 
-def bias_attention_runs(n_tiles: int, kv_heads: int, head_chunks: int, max_keys: int) -> int:
+def bias_attention_runs(n_tiles: int, kv_heads: int, head_chunks: int, max_keys: int, waves: int = 4) -> int:
     """Into how many runs the keys of a tile are cut: none while the tiles alone fill the chip's 256 compute
-    units or the keys are few, else towards two workgroups a unit, a run being at least ``RUN_KEYS`` keys."""
+    units or the keys are few, else towards 2,048 wavefronts, a run being at least ``RUN_KEYS`` keys."""
     blocks = max(1, n_tiles * kv_heads * head_chunks)
     if blocks >= 256 or max_keys < 2 * RUN_KEYS:
         return 1
-    return max(1, min(64, 512 // blocks, max_keys // RUN_KEYS))
+    return max(1, min(64, 2048 // (blocks * waves), max_keys // RUN_KEYS))
 
 
 def bias_attention_rows() -> int:
@@ -230,13 +230,14 @@ def kv_store(qkv: torch.Tensor, k_off: int, v_off: int, slot_mapping: torch.Tens
 def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int, scale: float,
                    temp_coef: float, temp_every: int, heads_per_chunk: int, n_runs: int = 1,
-                   workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   workspace: Optional[torch.Tensor] = None, waves: int = 4) -> torch.Tensor:
     """Causal attention of the query heads in the first ``H * dk`` columns of ``qkv`` over the paged cache.
     ``tiles`` int32 [n, 4]: (sequence, first row, tokens, -) with tokens * heads of a chunk <= 16, the tokens of a
     tile being consecutive ones of one sequence; ``positions`` int32 [T] the position of every row;
     ``bias`` float32 [distances, H] or None; ``out`` [T, H * dv].  With ``n_runs`` > 1 the keys of every tile are
     cut into that many runs, which meet in ``workspace`` (float32, at least T * H * n_runs * (dv + 2)) and are merged
-    by a second kernel."""
+    by a second kernel.  ``waves`` (1 to 4): wavefronts of a workgroup, four rows each; fewer than four only where no
+    tile has more rows than they take."""
     T, width = qkv.shape
     pages, G, ps, dk = kpool.shape
     dv = vpool.shape[3]
@@ -258,13 +259,14 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _need(dv <= 256, "values of more than 256 channels are not compiled")
     _need(1 <= heads_per_chunk <= 16, "heads_per_chunk")
     _need(1 <= n_runs <= 64, "n_runs")
+    _need(1 <= waves <= 4, "waves")
     if n_runs > 1:
         _need(workspace is not None and workspace.is_cuda and workspace.dtype == torch.float32 and workspace.is_contiguous()
               and workspace.numel() >= T * H * n_runs * (dv + 2), "the runs need a float32 workspace of T * H * n_runs * (dv + 2)")
     err = bias_attention_lib().ni_bias_attention(_ptr(qkv), width, _ptr(kpool), _ptr(vpool), _ptr(block_table),
                                                  block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions), _ptr(bias), distances,
                                                  _ptr(out), H, G, dk, dv, ps, _float(scale), _float(temp_coef), int(temp_every),
-                                                 heads_per_chunk, n_runs, _ptr(workspace if n_runs > 1 else None), T,
+                                                 heads_per_chunk, n_runs, _ptr(workspace if n_runs > 1 else None), T, waves,
                                                  dtype_code(qkv.dtype), _stream())
     if err == -2:
         raise KernelError(f"keys of {dk} and values of {dv} channels do not fit the kernel's staging memory")

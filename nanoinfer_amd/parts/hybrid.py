@@ -211,10 +211,13 @@ class BiasAttention(Part):
             raise K.KernelError("this step was recorded without the tiles of its tokens")
         out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
         chunks = -(-(self.H // self.G) // self.heads_per_chunk)
-        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, ctx.max_context)
+        # a step of single tokens has tiles of one token: its rows are the heads of a chunk, four a wavefront
+        rows = min(self.tile_tokens, ctx.max_q_len) * self.heads_per_chunk
+        waves = min(4, -(-rows // 4))
+        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, ctx.max_context, waves)
         ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
         K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H, self.scale,
-                         self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws)
+                         self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves)
         return K.linear(out, self.w_o, out_dtype=torch.float32)
 
 

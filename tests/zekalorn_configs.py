@@ -37,7 +37,7 @@ def model(width, vocab, layers, loop=None, side=None, max_positions=512, scale=3
 
 # one mechanism at a time
 ATTENTION_ONLY = model(64, 97, [(attention(4, 2, 16, 24, 0.5, bias_max=40.0, q_temp=(0.5, 8), bias_rows=12), None)])
-ATTENTION_PLAIN = model(48, 50, [(attention(3, 3, 16, 16, 0.25), None)])
+ATTENTION_PLAIN = model(48, 50, [(attention(3, 3, 18, 10, 0.25), None)])     # sizes that are no whole 16-byte pieces
 DELTA_ONLY = model(64, 97, [(delta(4, 2, 16, 24, 3, 8, 12), None)])
 DELTA_NO_CONV = model(40, 61, [(delta(2, 1, 20, 8, 1, 5, 7), None)])
 DENSE_FF = model(64, 97, [(attention(2, 1, 32, 32, 0.2), dense(88))])
