@@ -27,6 +27,20 @@
 #define PARTS 16
 #endif
 
+// Sum over the PARTS neighbouring lanes that hold one column (PARTS a power of two up to 16, aligned: they lie in
+// one row of sixteen lanes), every lane getting the total, by data-parallel moves inside the row: pairs, quads, the
+// mirrored half, the mirrored row.  No trip through the LDS crossbar stands in the recurrence's chain.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int N> __device__ __forceinline__ float parts_sum(float v) {
+    if constexpr (N >= 2) v += dpp_move<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+    if constexpr (N >= 4) v += dpp_move<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+    if constexpr (N >= 8) v += dpp_move<0x141>(v);      // row_half_mirror: lane i <-> 7 - i of its eight
+    if constexpr (N >= 16) v += dpp_move<0x140>(v);     // row_mirror: lane i <-> 15 - i of its sixteen
+    return v;
+}
+
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float silu_f(float z) { return z * sigmoid_f(z); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
@@ -187,12 +201,9 @@ delta_rule_kernel(const float* __restrict__ prep, float* __restrict__ state, con
                 b += S[i] * q;
                 kq += k[i] * q;
             }
-#pragma unroll
-            for (int off = 1; off < PARTS; off <<= 1) {
-                a += __shfl_xor(a, off, WAVE);
-                b += __shfl_xor(b, off, WAVE);
-                kq += __shfl_xor(kq, off, WAVE);
-            }
+            a = parts_sum<PARTS>(a);
+            b = parts_sum<PARTS>(b);
+            kq = parts_sum<PARTS>(kq);
             const float u = r[3 * DK + COLS] * (r[3 * DK + lcol] - a);
 #pragma unroll
             for (int i = 0; i < KPT; ++i) S[i] += k[i] * u;
@@ -235,7 +246,8 @@ NI_EXPORT int ni_delta_prepare(const void* proj, const void* low, const void* co
     if (dk != KPT * PARTS) return -1;
     const int C = 2 * G * dk + H * dv;
     if (dk > 256) return -2;
-    delta_prepare_kernel<<<dim3(T, 2 * G + H), 256, 0, stream>>>((const float*)proj, (const float*)low, (const float*)conv,
+    const int widest = std::max(dk, std::min(dv, 256));
+    delta_prepare_kernel<<<dim3(T, 2 * G + H), (widest + 63) / 64 * 64, 0, stream>>>((const float*)proj, (const float*)low, (const float*)conv,
                                                   (const float*)a_log, (const float*)dt_bias, (const float*)state,
                                                   (const int32_t*)seq_of_token, (const int32_t*)q_start,
                                                   (const int32_t*)state_slot, (float*)prep, G, H, dk, dv, taps, proj_cols,
