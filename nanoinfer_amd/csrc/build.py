@@ -126,7 +126,7 @@ SKINNY = ("ni_skinny_gemm", ["gemv.hip"], {})
 STREAM_OPS = ("ni_stream_ops", ["stream_ops.hip"], {})
 BIAS_ATTENTION = ("ni_bias_attention", ["bias_attention.hip"], {})
 COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
-COMMON_DELTA_KEY_SIZES = (16, 32, 48, 64, 96, 128)
+COMMON_DELTA_KEY_SIZES = (16, 20, 32, 48, 64, 96, 128)
 
 
 def delta_rule_split(key_size: int):
