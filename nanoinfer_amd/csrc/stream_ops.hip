@@ -156,42 +156,52 @@ NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int
 // z float32 [T, E]: the `top` largest logits of a row (the lower index on equal logits), their softmax
 // among themselves.  chosen int32 [T, top], mix float32 [T, top], and (if asked for) the same as a row
 // over all experts, zero where an expert was not chosen.
+// One wavefront a row: a lane keeps the logits of experts lane, lane + 64, ...; each of the `top` rounds finds the
+// largest logit not yet taken (the lowest index among equal ones) by two butterflies over the lanes.
 __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen, float* __restrict__ mix,
                                  float* __restrict__ mix_all, int T, int E, int top) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= T) return;
+    const int t = blockIdx.x, lane = threadIdx.x;
     const float* row = z + static_cast<size_t>(t) * E;
     int32_t* c = chosen + static_cast<size_t>(t) * top;
     float* m = mix + static_cast<size_t>(t) * top;
     float best = 0.f, total = 0.f;
-    for (int k = 0; k < top; ++k) {
-        int at = -1;
-        float v = 0.f;
-        for (int e = 0; e < E; ++e) {
-            bool taken = false;
-            for (int j = 0; j < k; ++j) taken |= (c[j] == e);
-            const float ze = row[e];
-            if (!taken && (at < 0 || ze > v)) { at = e; v = ze; }
-        }
-        c[k] = at;
-        if (k == 0) best = v;
-        const float w = expf(v - best);
-        m[k] = w;
-        total += w;
+    unsigned taken_mask = 0;        // bit j: this lane's expert lane + 64 j has been chosen
+    if (mix_all) {                  // zeros first; the fence lets them land before lane 0 writes the chosen ones at the end
+        for (int e = lane; e < E; e += WAVE) mix_all[static_cast<size_t>(t) * E + e] = 0.f;
+        __threadfence_block();
     }
-    if (mix_all)
-        for (int e = 0; e < E; ++e) mix_all[static_cast<size_t>(t) * E + e] = 0.f;
     for (int k = 0; k < top; ++k) {
-        const float w = m[k] / total;
-        m[k] = w;
-        if (mix_all) mix_all[static_cast<size_t>(t) * E + c[k]] = w;
+        float v = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane; e < E; e += WAVE) {
+            const bool taken = (taken_mask >> (e / WAVE)) & 1u;
+            float ze = row[e];
+            if (!(ze == ze)) ze = -INFINITY;       // a logit that is no number is never preferred
+            if (!taken && (at == 0x7fffffff || ze > v)) { at = e; v = ze; }
+        }
+        const float vmax = wave_max(v);
+        int cand = (at != 0x7fffffff && v == vmax) ? at : 0x7fffffff;
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, WAVE));
+        if (k == 0) best = vmax;
+        const float w = expf(vmax - best);
+        total += w;
+        if (cand % WAVE == lane) taken_mask |= 1u << (cand / WAVE);
+        if (lane == 0) { c[k] = cand; m[k] = w; }
+    }
+    if (lane == 0) {
+        for (int k = 0; k < top; ++k) {
+            const float w = m[k] / total;
+            m[k] = w;
+            if (mix_all) mix_all[static_cast<size_t>(t) * E + c[k]] = w;
+        }
     }
 }
 
 NI_EXPORT int ni_route_top(const void* z, void* chosen, void* mix, void* mix_all, int T, int E, int top, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (top < 1 || top > E) return -1;
-    route_top_kernel<<<blocks_of(T, 64), 64, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top);
+    if (top < 1 || top > E || E > 32 * WAVE) return -1;
+    route_top_kernel<<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top);
     return NI_LAUNCH_RESULT();
 }
 
