@@ -465,7 +465,7 @@ def main() -> int:
                          "the pool holds 2,048 more for every request")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the further points")
     ap.add_argument("--no-further", action="store_true",
-                    help="skip the points beyond the contract's: contexts of 8k and 32k, float32, the 3B shape")
+                    help="skip the points beyond the default line's: contexts of 8k and 32k, float32, the 3B shape")
     ap.add_argument("--only", default=None, choices=["zekalorn", "llama"], help="hybrid: measure one of the two models")
     ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid"],
                     help="steps: the decode step and prefill of the result line's contract (default); "

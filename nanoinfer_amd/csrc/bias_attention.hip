@@ -102,9 +102,10 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
                       const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
                       int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk, int n_runs,
-                      float* __restrict__ partial, bool k_pieces, bool v_pieces) {
-    extern __shared__ float lds[];
-    const int dkp = dk + 1;                       // a lane reads its key's row: odd strides spread the banks
+                      float* __restrict__ partial, bool k_pieces, bool v_pieces, int dkp) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    // a lane reads its key's row: the stride is the row plus four floats where rows are whole 16-byte pieces (read
+    // as such), plus one otherwise; both spread the lanes over the banks
     float* Qs = lds;                              // [ROWS][dk]
     float* Ks = Qs + ROWS * dk;                   // [KEYS][dkp]
     float* Vs = Ks + KEYS * dkp;                  // [KEYS][dv]
@@ -160,10 +161,21 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
         for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) s[rr] = 0.f;
         const float* krow = Ks + lane * dkp;
         const float* qrow = Qs + wave * ROWS_PER_WAVE * dk;
-        for (int c = 0; c < dk; ++c) {
-            const float kv = krow[c];
+        if (dkp == dk + 4) {
+            for (int c = 0; c < dk; c += 4) {
+                const float4 kv = *reinterpret_cast<const float4*>(krow + c);
 #pragma unroll
-            for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) s[rr] += qrow[rr * dk + c] * kv;
+                for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
+                    const float4 q = *reinterpret_cast<const float4*>(qrow + rr * dk + c);
+                    s[rr] += q.x * kv.x + q.y * kv.y + q.z * kv.z + q.w * kv.w;
+                }
+            }
+        } else {
+            for (int c = 0; c < dk; ++c) {
+                const float kv = krow[c];
+#pragma unroll
+                for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) s[rr] += qrow[rr * dk + c] * kv;
+            }
         }
         const int key = k0 + lane;
         float* prow = Ps + wave * ROWS_PER_WAVE * KEYS;
@@ -195,10 +207,13 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
                 float add[ROWS_PER_WAVE];
 #pragma unroll
                 for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) add[rr] = 0.f;
-                for (int j = 0; j < KEYS; ++j) {
-                    const float vv = Vs[j * dv + c];
+                for (int j = 0; j < KEYS; j += 4) {
+                    const float v0 = Vs[j * dv + c], v1 = Vs[(j + 1) * dv + c], v2 = Vs[(j + 2) * dv + c], v3 = Vs[(j + 3) * dv + c];
 #pragma unroll
-                    for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) add[rr] += prow[rr * KEYS + j] * vv;
+                    for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
+                        const float4 p = *reinterpret_cast<const float4*>(prow + rr * KEYS + j);
+                        add[rr] += p.x * v0 + p.y * v1 + p.z * v2 + p.w * v3;
+                    }
                 }
 #pragma unroll
                 for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) acc[rr][cc] = acc[rr][cc] * alpha[rr] + add[rr];
@@ -270,7 +285,8 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
     if (n_tiles <= 0) return 0;
     if (dv > MAX_VCHUNKS * WAVE || H % G || heads_per_chunk < 1 || heads_per_chunk > ROWS) return -1;
     const int group = H / G;
-    const size_t lds = (static_cast<size_t>(ROWS) * dk + static_cast<size_t>(KEYS) * (dk + 1) + static_cast<size_t>(KEYS) * dv +
+    const int dkp = dk % 4 == 0 ? dk + 4 : dk + 1;
+    const size_t lds = (static_cast<size_t>(ROWS) * dk + static_cast<size_t>(KEYS) * dkp + static_cast<size_t>(KEYS) * dv +
                         WAVES * ROWS_PER_WAVE * KEYS) * sizeof(float);
     if (lds > 160 * 1024) return -2;
     if (n_runs < 1 || (n_runs > 1 && !partial) || waves < 1 || waves > WAVES) return -1;
@@ -288,7 +304,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<float><<<grid, waves * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp);
         if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv);
     } else {
         static size_t allowed = 48 * 1024;
@@ -298,7 +314,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<bf16_t><<<grid, waves * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp);
         if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv);
     }
     return NI_LAUNCH_RESULT();

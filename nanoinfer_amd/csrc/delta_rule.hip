@@ -189,19 +189,22 @@ delta_rule_kernel(const float* __restrict__ prep, float* __restrict__ state, con
         if (more) fetch(t0 + CHUNK);
         const float* cur = buf[which];
         const int count = min(CHUNK, n - t0);
+        // unrolled, so that the reads from LDS and the products that do not wait for the memory (k . q) of the next
+        // tokens stand ahead of the chain S -> S^T k -> u -> S that every token has to wait for
+#pragma unroll 4
         for (int tt = 0; tt < count; ++tt) {
             const float* r = cur + tt * ROW;
-            float a = 0.f, b = 0.f, kq = 0.f, k[KPT];
+            float a = 0.f, a1 = 0.f, b = 0.f, kq = 0.f, k[KPT];
 #pragma unroll
             for (int i = 0; i < KPT; ++i) {
                 const float q = r[part * KPT + i];
                 k[i] = r[DK + part * KPT + i];
                 S[i] *= r[2 * DK + part * KPT + i];
-                a += S[i] * k[i];
+                if (i & 1) a1 += S[i] * k[i]; else a += S[i] * k[i];      // two chains of half the length
                 b += S[i] * q;
                 kq += k[i] * q;
             }
-            a = parts_sum<PARTS>(a);
+            a = parts_sum<PARTS>(a + a1);
             b = parts_sum<PARTS>(b);
             kq = parts_sum<PARTS>(kq);
             const float u = r[3 * DK + COLS] * (r[3 * DK + lcol] - a);
