@@ -2,12 +2,14 @@
 //
 // Per head, with S [key channel, value channel] float32 carried from token to token:
 //     S <- diag(g_t) S;   u_t = beta_t (v_t - S^T k_t);   S <- S + k_t u_t^T;   o_t = S^T q_t
-// Four kernels:
+// Six kernels:
 //   delta_prepare      per token, in parallel: the short causal convolutions of q, k, v with silu, the unit
 //                      norms of q and k, beta = sigmoid, g = exp(-exp(A) softplus(z + dt)), the output gate
 //   conv_state_update  per sequence: the last taps - 1 inputs of the convolutions, kept for the next step
 //   delta_rule         per (sequence, head, group of value channels): the recurrence over the step's tokens
 //   headnorm_gate      o / rms(o) * w * gate per head, rounded to the compute type for the output product
+//   delta_chunk_prepare, delta_chunk_scan   the same recurrence for portions of prompts, sixteen tokens at a
+//                      time on the matrix cores (described above them)
 //
 // The columns of S are independent of one another: u_t[j] and o_t[j] need column j alone.  A column is
 // held by PARTS neighbouring lanes, KPT key channels each, in registers for the whole step; the three
@@ -70,7 +72,7 @@ __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float
                                      const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
                                      const int32_t* __restrict__ state_slot, float* __restrict__ prep,
                                      int G, int H, int dk, int dv, int taps, int proj_cols, size_t state_stride,
-                                     size_t conv_off) {
+                                     size_t conv_off, int log_decay) {
     __shared__ float scratch[16];
     const int t = blockIdx.x, unit = blockIdx.y;
     const int s = seq_of_token[t];
@@ -104,7 +106,8 @@ __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float
     const float rate = expf(a_log[h]);
     for (int j = threadIdx.x; j < dk; j += blockDim.x) {
         const float z = lrow[h * dk + j] + dt_bias[h * dk + j];
-        out[C + H + h * dk + j] = expf(-rate * (z > 20.f ? z : log1pf(expf(z))));
+        const float lg = -rate * (z > 20.f ? z : log1pf(expf(z)));
+        out[C + H + h * dk + j] = log_decay ? lg : expf(lg);      // the chunked form sums logarithms
     }
     if (threadIdx.x == 0) out[C + h] = 1.0f / (1.0f + expf(-prow[C + h]));
 }
@@ -222,6 +225,197 @@ delta_rule_kernel(const float* __restrict__ prep, float* __restrict__ state, con
     }
 }
 
+// ------------------------------------------------------------------ sixteen tokens at a time
+// Within a run of C = 16 tokens that starts from the memory S0, with L_t the sum of the logarithms of the decays
+// of the run's tokens up to t (a vector over the key channels):
+//     u_t + beta_t sum_{s<t} A_ts u_s = beta_t (v_t - S0^T (e^{L_t} k_t)),   A_ts = sum_c k_t[c] k_s[c] e^{L_t[c] - L_s[c]}
+//     o_t = S0^T (e^{L_t} q_t) + sum_{s<=t} P_ts u_s,                        P_ts = sum_c q_t[c] k_s[c] e^{L_t[c] - L_s[c]}
+//     S_C = diag(e^{L_C}) S0 + sum_s (e^{L_C - L_s} k_s) u_s^T
+// Every exponent is a difference that is at most zero: nothing is divided by a decay, however small it gets.
+// A, P, the inverse Tm = (I + diag(beta) tril(A, -1))^-1 diag(beta) and the three scaled copies of k and q do not
+// depend on the memory: delta_chunk_prepare makes them for all runs of the step at once.  What is left for the
+// chain from run to run is five small matrix products,
+//     W = V - Kt S0;  U = Tm W;  O = Qt S0 + P U;  S <- diag(e^{L_C}) S0 + Kb^T U,
+// which delta_chunk_scan does with v_mfma_f32_16x16x4_f32 (true 32-bit products and sums), one wavefront a
+// (sequence, head, sixteen value channels) with its [DK, 16] piece of S in the accumulators' layout for the whole
+// step.  A lane of that layout holds channels 4 (lane / 16) + r, r = 0..3, of each sixteen; as the second operand
+// of a product over channels the four registers are used one after the other, and the first operand is read in
+// the matching order (channel 4 (lane / 16) + r at step r), so that S never moves between layouts.
+// Tokens past a sequence's end count as k = q = v = 0, beta = 0, decay 1: they leave S as it is.
+// Runs are stored by slot = q_start / 16 + sequence + run: no two sequences of a step share one.
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+constexpr int RUN = 16;
+
+__host__ __device__ constexpr int chunk_floats(int dk) { return 3 * RUN * dk + 2 * RUN * RUN + dk; }
+
+__global__ void __launch_bounds__(256)
+delta_chunk_prepare_kernel(const float* __restrict__ prep, float* __restrict__ chunks, const int32_t* __restrict__ q_start,
+                           const int32_t* __restrict__ q_len, int G, int H, int dv) {
+    constexpr int DK = KPT * PARTS, LD = DK + 1;
+    __shared__ float Ls[RUN * LD], ks[RUN * LD], qs[RUN * LD], As[RUN * (RUN + 1)], betas[RUN];
+    const int s = blockIdx.x, h = blockIdx.z;
+    const int n = q_len[s], first = q_start[s];
+    const int t0 = blockIdx.y * RUN;
+    if (t0 >= n) return;
+    const int g = h / (H / G);
+    const int QK = 2 * G * DK, C = QK + H * dv;
+    const int prep_cols = C + H + H * DK + H * dv;
+    const size_t slot = static_cast<size_t>(first / RUN + s + blockIdx.y);
+    float* out = chunks + (slot * H + h) * chunk_floats(DK);
+    const float* rows = prep + static_cast<size_t>(first + t0) * prep_cols;
+    for (int e = threadIdx.x; e < RUN * DK; e += 256) {
+        const int t = e / DK, c = e % DK;
+        const bool valid = t0 + t < n;
+        const float* row = rows + static_cast<size_t>(t) * prep_cols;
+        Ls[t * LD + c] = valid ? row[C + H + h * DK + c] : 0.f;
+        ks[t * LD + c] = valid ? row[G * DK + g * DK + c] : 0.f;
+        qs[t * LD + c] = valid ? row[g * DK + c] : 0.f;
+    }
+    if (threadIdx.x < RUN) betas[threadIdx.x] = t0 + threadIdx.x < n ? rows[static_cast<size_t>(threadIdx.x) * prep_cols + C + h] : 0.f;
+    __syncthreads();
+    if (threadIdx.x < DK) {
+        float run = 0.f;
+        for (int t = 0; t < RUN; ++t) {
+            run += Ls[t * LD + threadIdx.x];
+            Ls[t * LD + threadIdx.x] = run;
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < RUN * DK; e += 256) {
+        const int t = e / DK, c = e % DK;
+        const float lt = Ls[t * LD + c], lc = Ls[(RUN - 1) * LD + c];
+        const float grow = expf(lt);
+        out[e] = grow * ks[t * LD + c];
+        out[RUN * DK + e] = grow * qs[t * LD + c];
+        out[2 * RUN * DK + e] = expf(lc - lt) * ks[t * LD + c];
+        if (t == RUN - 1) out[3 * RUN * DK + 2 * RUN * RUN + c] = grow;
+    }
+    {
+        const int t = threadIdx.x / RUN, j = threadIdx.x % RUN;
+        float a = 0.f, p = 0.f;
+        if (j <= t) {
+            for (int c = 0; c < DK; ++c) {
+                const float w = expf(Ls[t * LD + c] - Ls[j * LD + c]) * ks[j * LD + c];
+                a += ks[t * LD + c] * w;
+                p += qs[t * LD + c] * w;
+            }
+        }
+        As[t * (RUN + 1) + j] = j < t ? a : 0.f;
+        out[3 * RUN * DK + RUN * RUN + t * RUN + j] = j <= t ? p : 0.f;
+    }
+    __syncthreads();
+    if (threadIdx.x < RUN) {
+        // column j of (I + diag(beta) tril(A, -1))^-1 diag(beta), from the top down
+        const int j = threadIdx.x;
+        float x[RUN];
+#pragma unroll
+        for (int t = 0; t < RUN; ++t) {
+            float acc = 0.f;
+#pragma unroll
+            for (int r = 0; r < t; ++r) acc += As[t * (RUN + 1) + r] * x[r];
+            x[t] = (t == j ? betas[j] : 0.f) - betas[t] * acc;
+        }
+#pragma unroll
+        for (int t = 0; t < RUN; ++t) out[3 * RUN * DK + t * RUN + j] = x[t];
+    }
+}
+
+// What a wavefront reads for one run of tokens: all of it is asked for one run ahead.
+template <int KT> struct RunOperands {
+    float4 kt[KT], qt[KT], dec[KT];      // rows (lane % 16) of Kt and Qt, channels 16 kt + 4 (lane / 16) + r; e^{L_C} of these
+    float kb[KT][4];                     // Kb of token 4 (lane / 16) + r, channel 16 kt + lane % 16
+    float4 tm, p;                        // row (lane % 16) of Tm and of P, columns 4 (lane / 16) + r
+    floatx4_t v;                         // v of token 4 (lane / 16) + r, the lane's value channel
+};
+
+__global__ void __launch_bounds__(64)
+delta_chunk_scan_kernel(const float* __restrict__ prep, const float* __restrict__ chunks, float* __restrict__ state,
+                        const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+                        const int32_t* __restrict__ state_slot, float* __restrict__ o, int G, int H, int dv,
+                        size_t state_stride) {
+    constexpr int DK = KPT * PARTS, KT = DK / RUN;
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int i = threadIdx.x & 15, g4 = threadIdx.x >> 4;
+    const int col = blockIdx.z * RUN + i;
+    const bool live = col < dv;
+    const int n = q_len[s], first = q_start[s];
+    if (n <= 0) return;
+    const int QK = 2 * G * DK, C = QK + H * dv;
+    const int prep_cols = C + H + H * DK + H * dv;
+    float* S_mem = state + static_cast<size_t>(state_slot[s]) * state_stride + (static_cast<size_t>(h) * dv + (live ? col : 0)) * DK + 4 * g4;
+    floatx4_t S[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) S[kt][r] = live ? S_mem[kt * RUN + r] : 0.f;
+    const float* base = chunks + (static_cast<size_t>(first / RUN + s) * H + h) * chunk_floats(DK);
+    const size_t per_run = static_cast<size_t>(H) * chunk_floats(DK);
+    const float* vcol = prep + static_cast<size_t>(first) * prep_cols + QK + h * dv + (live ? col : 0);
+
+    auto fetch = [&](RunOperands<KT>& x, int run) {
+        const float* ch = base + per_run * run;
+        const int t0 = run * RUN;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            x.kt[kt] = *reinterpret_cast<const float4*>(ch + i * DK + kt * RUN + 4 * g4);
+            x.qt[kt] = *reinterpret_cast<const float4*>(ch + RUN * DK + i * DK + kt * RUN + 4 * g4);
+            x.dec[kt] = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + 2 * RUN * RUN + kt * RUN + 4 * g4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) x.kb[kt][r] = ch[2 * RUN * DK + (4 * g4 + r) * DK + kt * RUN + i];
+        }
+        x.tm = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + i * RUN + 4 * g4);
+        x.p = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + RUN * RUN + i * RUN + 4 * g4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int tok = t0 + 4 * g4 + r;
+            x.v[r] = (live && tok < n) ? vcol[static_cast<size_t>(tok) * prep_cols] : 0.f;
+        }
+    };
+    auto at = [](const float4& f, int r) { return r == 0 ? f.x : r == 1 ? f.y : r == 2 ? f.z : f.w; };
+
+    const int runs = (n + RUN - 1) / RUN;
+    RunOperands<KT> cur, nxt;
+    fetch(cur, 0);
+    for (int run = 0; run < runs; ++run) {
+        if (run + 1 < runs) fetch(nxt, run + 1);
+        floatx4_t w = {0.f, 0.f, 0.f, 0.f}, out = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                w = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.kt[kt], r), S[kt][r], w, 0, 0, 0);
+                out = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.qt[kt], r), S[kt][r], out, 0, 0, 0);
+            }
+        w = cur.v - w;
+        floatx4_t u = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) u = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.tm, r), w[r], u, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) out = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.p, r), u[r], out, 0, 0, 0);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) S[kt][r] *= at(cur.dec[kt], r);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) S[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.kb[kt][r], u[r], S[kt], 0, 0, 0);
+        }
+        if (live) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int tok = run * RUN + 4 * g4 + r;
+                if (tok < n) o[(static_cast<size_t>(first) + tok) * (H * dv) + h * dv + col] = out[r];
+            }
+        }
+        cur = nxt;
+    }
+    if (live) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) S_mem[kt * RUN + r] = S[kt][r];
+    }
+}
+
 // y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w * gate[t, h, :]; one wavefront a (token, head)
 template <typename T>
 __global__ void headnorm_gate_kernel(const float* __restrict__ o, const float* __restrict__ gate, size_t gate_stride,
@@ -244,7 +438,7 @@ NI_EXPORT int ni_delta_key_size() { return KPT * PARTS; }
 NI_EXPORT int ni_delta_prepare(const void* proj, const void* low, const void* conv, const void* a_log, const void* dt_bias,
                                void* state, const void* seq_of_token, const void* q_start, const void* q_len,
                                const void* state_slot, void* prep, int T, int B, int G, int H, int dk, int dv, int taps,
-                               int proj_cols, size_t state_stride, size_t conv_off, hipStream_t stream) {
+                               int proj_cols, size_t state_stride, size_t conv_off, int log_decay, hipStream_t stream) {
     if (T <= 0) return 0;
     if (dk != KPT * PARTS) return -1;
     const int C = 2 * G * dk + H * dv;
@@ -254,7 +448,7 @@ NI_EXPORT int ni_delta_prepare(const void* proj, const void* low, const void* co
                                                   (const float*)a_log, (const float*)dt_bias, (const float*)state,
                                                   (const int32_t*)seq_of_token, (const int32_t*)q_start,
                                                   (const int32_t*)state_slot, (float*)prep, G, H, dk, dv, taps, proj_cols,
-                                                  state_stride, conv_off);
+                                                  state_stride, conv_off, log_decay);
     if (taps > 1) {
         dim3 grid(B, std::max(1, std::min(64, (C + 255) / 256)));
         conv_state_update_kernel<<<grid, 256, 0, stream>>>((const float*)proj, (float*)state, (const int32_t*)q_start,
@@ -264,16 +458,36 @@ NI_EXPORT int ni_delta_prepare(const void* proj, const void* low, const void* co
     return NI_LAUNCH_RESULT();
 }
 
-NI_EXPORT int ni_delta_rule(const void* prep, void* state, const void* q_start, const void* q_len, const void* state_slot,
-                            void* o, const void* norm_w, void* y, int T, int B, int G, int H, int dk, int dv, float eps,
-                            size_t state_stride, int dtype, hipStream_t stream) {
+// floats of scratch that the chunked form needs per run of sixteen tokens and head (0: this key size has no such form);
+// a step of T tokens in B sequences has at most T / 16 + B + 1 run slots
+NI_EXPORT int ni_delta_run_floats() { return (KPT * PARTS) % RUN ? 0 : chunk_floats(KPT * PARTS); }
+
+// chunks: null for the token-by-token kernel (prep then holds the decays), else scratch for the chunked form
+// (prep then holds the decays' logarithms); max_q_len is the longest portion of the step
+NI_EXPORT int ni_delta_rule(const void* prep, void* chunks, void* state, const void* q_start, const void* q_len,
+                            const void* state_slot, void* o, const void* norm_w, void* y, int T, int B, int max_q_len, int G,
+                            int H, int dk, int dv, float eps, size_t state_stride, int dtype, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
     if (dk != KPT * PARTS) return -1;
-    constexpr int COLS = 256 / PARTS;
-    dim3 grid(B, H, (dv + COLS - 1) / COLS);
-    delta_rule_kernel<<<grid, 256, 0, stream>>>((const float*)prep, (float*)state, (const int32_t*)q_start,
-                                                (const int32_t*)q_len, (const int32_t*)state_slot, (float*)o, G, H, dv,
-                                                state_stride);
+    if (chunks) {
+        if constexpr ((KPT * PARTS) % RUN == 0) {
+            if (max_q_len < 1) return -1;
+            const int runs = (max_q_len + RUN - 1) / RUN;
+            delta_chunk_prepare_kernel<<<dim3(B, runs, H), 256, 0, stream>>>((const float*)prep, (float*)chunks, (const int32_t*)q_start,
+                                                                             (const int32_t*)q_len, G, H, dv);
+            delta_chunk_scan_kernel<<<dim3(B, H, (dv + RUN - 1) / RUN), 64, 0, stream>>>(
+                (const float*)prep, (const float*)chunks, (float*)state, (const int32_t*)q_start, (const int32_t*)q_len,
+                (const int32_t*)state_slot, (float*)o, G, H, dv, state_stride);
+        } else {
+            return -3;
+        }
+    } else {
+        constexpr int COLS = 256 / PARTS;
+        dim3 grid(B, H, (dv + COLS - 1) / COLS);
+        delta_rule_kernel<<<grid, 256, 0, stream>>>((const float*)prep, (float*)state, (const int32_t*)q_start,
+                                                    (const int32_t*)q_len, (const int32_t*)state_slot, (float*)o, G, H, dv,
+                                                    state_stride);
+    }
     const int C = 2 * G * dk + H * dv;
     const int prep_cols = C + H + H * dk + H * dv;
     const float* gate = (const float*)prep + C + H + H * dk;

@@ -151,17 +151,24 @@ def experts_few(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chose
 
 # ------------------------------------------------------------------ gated delta rule
 
+DELTA_RUN_FROM = 16      # a step whose longest portion has this many tokens goes in runs of sixteen
+
+
 def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                norm_w: torch.Tensor, state: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor,
                q_len: torch.Tensor, state_slot: torch.Tensor, G: int, H: int, dk: int, dv: int, taps: int, eps: float,
-               out_dtype: torch.dtype) -> torch.Tensor:
+               out_dtype: torch.dtype, max_q_len: int = 1) -> torch.Tensor:
     """One step of the gated delta rule with a decay per key channel for all sequences of the step.
 
     ``proj`` float32 [T, >= C + H] holds q [G*dk] | k [G*dk] | v [H*dv] | b [H] as projected (C the first
     three); ``low`` float32 [T, H*dk + H*dv] the decay's and the output gate's pre-activations; ``conv``
     float32 [C, taps]; ``state`` float32 [slots, H*dv*dk + (taps-1)*C]: the memory of every head (stored
     [head, value channel, key channel]) and the convolutions' last inputs, both moved on by this call.
-    Returns the normalised, gated read-out [T, H*dv] in ``out_dtype``."""
+    Returns the normalised, gated read-out [T, H*dv] in ``out_dtype``.
+
+    ``max_q_len`` is the longest portion of the step (a host number).  From ``DELTA_RUN_FROM`` tokens on, and
+    where the key size is a multiple of 16, the step goes sixteen tokens at a time on the matrix cores (in
+    float32 as well); otherwise token by token.  Both compute the same recurrence and differ by rounding."""
     T, proj_cols = proj.shape
     B = q_start.shape[0]
     C = 2 * G * dk + H * dv
@@ -182,13 +189,19 @@ def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log:
     lib = delta_rule_lib(dk)
     prep = torch.empty(T, C + H + H * dk + H * dv, dtype=torch.float32, device=proj.device)
     stride = state.shape[1]
+    run_floats = int(lib.ni_delta_run_floats()) if max_q_len >= DELTA_RUN_FROM else 0
+    chunks = None
+    if run_floats:
+        _need(max_q_len <= T, "max_q_len is larger than the step")
+        chunks = torch.empty((T // 16 + B + 1) * H * run_floats, dtype=torch.float32, device=proj.device)
     _check(lib.ni_delta_prepare(_ptr(proj), _ptr(low), _ptr(conv), _ptr(a_log), _ptr(dt_bias), _ptr(state), _ptr(seq_of_token),
                                 _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(prep), T, B, G, H, dk, dv, taps, proj_cols,
-                                _size_t(stride), _size_t(conv_off), _stream()), "delta_prepare")
+                                _size_t(stride), _size_t(conv_off), int(chunks is not None), _stream()), "delta_prepare")
     o = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
     y = torch.empty(T, H * dv, dtype=out_dtype, device=proj.device)
-    _check(lib.ni_delta_rule(_ptr(prep), _ptr(state), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(o), _ptr(norm_w),
-                             _ptr(y), T, B, G, H, dk, dv, _float(eps), _size_t(stride), dtype_code(out_dtype), _stream()),
+    _check(lib.ni_delta_rule(_ptr(prep), _ptr(chunks), _ptr(state), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(o),
+                             _ptr(norm_w), _ptr(y), T, B, int(max_q_len), G, H, dk, dv, _float(eps), _size_t(stride),
+                             dtype_code(out_dtype), _stream()),
            "delta_rule")
     return y
 

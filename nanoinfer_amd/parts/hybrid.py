@@ -305,7 +305,7 @@ class ChannelDelta(Part):
         seq = ctx.per_seq
         y = K.delta_rule(proj, low, self.conv, self.a_log, self.dt_bias, self.norm, cache.state, ctx.seq_of_token,
                          seq.q_start, seq.q_len, seq.state_slot, self.G, self.H, self.dk, self.dv, self.taps, self.eps,
-                         self.rt.dtype)
+                         self.rt.dtype, max_q_len=ctx.max_q_len)
         return K.linear(y, self.w_o, out_dtype=torch.float32)
 
 

@@ -335,6 +335,76 @@ def test_few_rows_and_many_rows_of_routed_experts_agree_with_the_plain_sum(dtype
         assert err < tol, (name, err)
 
 
+# ------------------------------------------------------------------ the delta rule's two kernels
+
+def _plain_delta_step(proj, low, conv, a_log, dt_bias, norm_w, state, starts, lens, slots, G, H, dk, dv, taps, eps):
+    """The delta rule's kernel interface in float64, token by token: the read-out rows and the new state."""
+    C = 2 * G * dk + H * dv
+    state = state.clone()
+    out = torch.zeros(proj.shape[0], H * dv, dtype=torch.float64)
+    silu = lambda z: z * torch.sigmoid(z)
+    for first, n, slot in zip(starts, lens, slots):
+        S = state[slot, : H * dv * dk].view(H, dv, dk).transpose(1, 2).clone()          # [H, dk, dv]
+        hist = state[slot, H * dv * dk:].view(taps - 1, C)
+        xs = torch.cat([hist, proj[first: first + n, :C]], dim=0)                         # [taps - 1 + n, C]
+        for i in range(n):
+            t = first + i
+            z = (xs[i: i + taps] * conv.t()).sum(dim=0)
+            a = silu(z)
+            q, k, v = a[: G * dk].view(G, dk), a[G * dk: 2 * G * dk].view(G, dk), a[2 * G * dk:].view(H, dv)
+            q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+            k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+            beta = torch.sigmoid(proj[t, C: C + H])
+            decay = torch.exp(-torch.exp(a_log).view(H, 1) * torch.nn.functional.softplus(low[t, : H * dk] + dt_bias).view(H, dk))
+            gate = torch.sigmoid(low[t, H * dk:]).view(H, dv)
+            for h in range(H):
+                g = h // (H // G)
+                S[h] = decay[h].view(dk, 1) * S[h]
+                u = beta[h] * (v[h] - S[h].t() @ k[g])
+                S[h] = S[h] + torch.outer(k[g], u)
+                o = S[h].t() @ q[g]
+                out[t, h * dv:(h + 1) * dv] = o / torch.sqrt((o * o).mean() + eps) * norm_w * gate[h]
+        state[slot, : H * dv * dk] = S.transpose(1, 2).reshape(-1)
+        state[slot, H * dv * dk:] = xs[n:].reshape(-1)
+    return out, state
+
+
+@pytest.mark.parametrize("decay", ["mild", "strong"])
+@pytest.mark.parametrize("G,H,dk,dv,taps", [(2, 4, 32, 24, 3), (1, 1, 16, 16, 2), (3, 3, 64, 40, 4), (1, 2, 128, 20, 2)])
+def test_delta_rule_in_runs_of_sixteen_and_token_by_token_agree_with_the_plain_recurrence(G, H, dk, dv, taps, decay):
+    """One step of unequal portions (1, 15, 16, 17 and 50 tokens: less than a run, a whole one, one more, and
+    several) from a state that is not zero, on slots in another order than the sequences.  With strong decays
+    (a channel keeps 1e-9 or less of itself per token) a form that divided by products of decays would overflow."""
+    from nanoinfer_amd import kernels as K
+    g = torch.Generator().manual_seed(dk + dv)
+    lens = [1, 15, 16, 17, 50]
+    starts = [sum(lens[:i]) for i in range(len(lens))]
+    slots = [3, 0, 4, 1, 6]
+    T, C = sum(lens), 2 * G * dk + H * dv
+    proj = torch.randn(T, C + H, generator=g, dtype=torch.float64) * 1.5
+    low = torch.randn(T, H * dk + H * dv, generator=g, dtype=torch.float64)
+    conv = torch.randn(C, taps, generator=g, dtype=torch.float64) * 0.7
+    a_log = torch.randn(H, generator=g, dtype=torch.float64) * 0.3 + (3.0 if decay == "strong" else -1.0)
+    dt_bias = torch.randn(H * dk, generator=g, dtype=torch.float64)
+    norm_w = torch.rand(dv, generator=g, dtype=torch.float64) + 0.5
+    state = torch.randn(7, H * dv * dk + (taps - 1) * C, generator=g, dtype=torch.float64) * 0.5
+    want, want_state = _plain_delta_step(proj, low, conv, a_log, dt_bias, norm_w, state, starts, lens, slots, G, H, dk, dv, taps, 1e-5)
+    dev = torch.device("cuda")
+    f32 = lambda t: t.to(dev, torch.float32).contiguous()
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    seq_of_token = i32([s for s, n in enumerate(lens) for _ in range(n)])
+    for what, longest in (("token by token", 1), ("runs of sixteen", max(lens))):
+        st = f32(state)
+        got = K.delta_rule(f32(proj), f32(low), f32(conv), f32(a_log), f32(dt_bias), f32(norm_w), st, seq_of_token, i32(starts),
+                           i32(lens), i32(slots), G, H, dk, dv, taps, 1e-5, torch.float32, max_q_len=longest)
+        err = float((got.double().cpu() - want).abs().max() / want.abs().max())
+        assert err < 2e-5, (what, "read-out", err)
+        err = float((st.double().cpu() - want_state).abs().max() / want_state.abs().max())
+        assert err < 2e-5, (what, "state", err)
+        untouched = [s for s in range(7) if s not in slots]
+        assert torch.equal(st.cpu()[untouched], state.float()[untouched]), what
+
+
 # ------------------------------------------------------------------ generation through the entry point
 
 @pytest.mark.parametrize("name", ["mixed", "loop_all"])
