@@ -236,7 +236,7 @@ delta_rule_kernel(const float* __restrict__ prep, float* __restrict__ state, con
 // depend on the memory: delta_chunk_prepare makes them for all runs of the step at once.  What is left for the
 // chain from run to run is five small matrix products,
 //     W = V - Kt S0;  U = Tm W;  O = Qt S0 + P U;  S <- diag(e^{L_C}) S0 + Kb^T U,
-// which delta_chunk_scan does with v_mfma_f32_16x16x4_f32 (true 32-bit products and sums), one wavefront a
+// which delta_chunk_scan does with v_mfma_f32_16x16x4_f32 (true 32-bit products and sums), one workgroup a
 // (sequence, head, sixteen value channels) with its [DK, 16] piece of S in the accumulators' layout for the whole
 // step.  A lane of that layout holds channels 4 (lane / 16) + r, r = 0..3, of each sixteen; as the second operand
 // of a product over channels the four registers are used one after the other, and the first operand is read in
@@ -321,47 +321,57 @@ delta_chunk_prepare_kernel(const float* __restrict__ prep, float* __restrict__ c
 }
 
 // What a wavefront reads for one run of tokens: all of it is asked for one run ahead.
-template <int KT> struct RunOperands {
-    float4 kt[KT], qt[KT], dec[KT];      // rows (lane % 16) of Kt and Qt, channels 16 kt + 4 (lane / 16) + r; e^{L_C} of these
-    float kb[KT][4];                     // Kb of token 4 (lane / 16) + r, channel 16 kt + lane % 16
+template <int KTW> struct RunOperands {
+    float4 kt[KTW], qt[KTW], dec[KTW];   // rows (lane % 16) of Kt and Qt, channels 16 kt + 4 (lane / 16) + r; e^{L_C} of these
+    float kb[KTW][4];                    // Kb of token 4 (lane / 16) + r, channel 16 kt + lane % 16
     float4 tm, p;                        // row (lane % 16) of Tm and of P, columns 4 (lane / 16) + r
     floatx4_t v;                         // v of token 4 (lane / 16) + r, the lane's value channel
 };
 
-__global__ void __launch_bounds__(64)
+// The key channels of a (head, sixteen value channels) are dealt to SCAN_WAVES wavefronts, sixteen at a time: each
+// keeps its channels' rows of S and makes its share of Kt S0 and Qt S0.  The shares meet in LDS once a run (two
+// buffers in turn, so one barrier a run is enough: a wavefront can be one run ahead of another, never two); every
+// wavefront then sums them in the same order, so all hold the same W and U, and moves its own rows of S on.
+constexpr int scan_waves(int kt) { return kt % 4 == 0 ? 4 : kt % 2 == 0 ? 2 : 1; }
+
+__global__ void __launch_bounds__(64 * scan_waves(KPT * PARTS / RUN > 0 ? KPT * PARTS / RUN : 1))
 delta_chunk_scan_kernel(const float* __restrict__ prep, const float* __restrict__ chunks, float* __restrict__ state,
                         const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
                         const int32_t* __restrict__ state_slot, float* __restrict__ o, int G, int H, int dv,
                         size_t state_stride) {
-    constexpr int DK = KPT * PARTS, KT = DK / RUN;
+    constexpr int DK = KPT * PARTS, KT = DK / RUN > 0 ? DK / RUN : 1, SW = scan_waves(KT), KTW = KT / SW;
+    __shared__ float shares[2][SW][2][4][WAVE];
     const int s = blockIdx.x, h = blockIdx.y;
-    const int i = threadIdx.x & 15, g4 = threadIdx.x >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
+    const int i = lane & 15, g4 = lane >> 4;
     const int col = blockIdx.z * RUN + i;
     const bool live = col < dv;
     const int n = q_len[s], first = q_start[s];
     if (n <= 0) return;
     const int QK = 2 * G * DK, C = QK + H * dv;
     const int prep_cols = C + H + H * DK + H * dv;
-    float* S_mem = state + static_cast<size_t>(state_slot[s]) * state_stride + (static_cast<size_t>(h) * dv + (live ? col : 0)) * DK + 4 * g4;
-    floatx4_t S[KT];
+    const int ch0 = wave * KTW * RUN;                  // the wavefront's first key channel
+    float* S_mem = state + static_cast<size_t>(state_slot[s]) * state_stride + (static_cast<size_t>(h) * dv + (live ? col : 0)) * DK + ch0 + 4 * g4;
+    floatx4_t S[KTW];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt)
+    for (int kt = 0; kt < KTW; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) S[kt][r] = live ? S_mem[kt * RUN + r] : 0.f;
     const float* base = chunks + (static_cast<size_t>(first / RUN + s) * H + h) * chunk_floats(DK);
     const size_t per_run = static_cast<size_t>(H) * chunk_floats(DK);
     const float* vcol = prep + static_cast<size_t>(first) * prep_cols + QK + h * dv + (live ? col : 0);
 
-    auto fetch = [&](RunOperands<KT>& x, int run) {
+    auto fetch = [&](RunOperands<KTW>& x, int run) {
         const float* ch = base + per_run * run;
         const int t0 = run * RUN;
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            x.kt[kt] = *reinterpret_cast<const float4*>(ch + i * DK + kt * RUN + 4 * g4);
-            x.qt[kt] = *reinterpret_cast<const float4*>(ch + RUN * DK + i * DK + kt * RUN + 4 * g4);
-            x.dec[kt] = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + 2 * RUN * RUN + kt * RUN + 4 * g4);
+        for (int kt = 0; kt < KTW; ++kt) {
+            const int c = ch0 + kt * RUN;
+            x.kt[kt] = *reinterpret_cast<const float4*>(ch + i * DK + c + 4 * g4);
+            x.qt[kt] = *reinterpret_cast<const float4*>(ch + RUN * DK + i * DK + c + 4 * g4);
+            x.dec[kt] = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + 2 * RUN * RUN + c + 4 * g4);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) x.kb[kt][r] = ch[2 * RUN * DK + (4 * g4 + r) * DK + kt * RUN + i];
+            for (int r = 0; r < 4; ++r) x.kb[kt][r] = ch[2 * RUN * DK + (4 * g4 + r) * DK + c + i];
         }
         x.tm = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + i * RUN + 4 * g4);
         x.p = *reinterpret_cast<const float4*>(ch + 3 * RUN * DK + RUN * RUN + i * RUN + 4 * g4);
@@ -374,43 +384,67 @@ delta_chunk_scan_kernel(const float* __restrict__ prep, const float* __restrict_
     auto at = [](const float4& f, int r) { return r == 0 ? f.x : r == 1 ? f.y : r == 2 ? f.z : f.w; };
 
     const int runs = (n + RUN - 1) / RUN;
-    RunOperands<KT> cur, nxt;
+    RunOperands<KTW> cur, nxt;
     fetch(cur, 0);
     for (int run = 0; run < runs; ++run) {
         if (run + 1 < runs) fetch(nxt, run + 1);
         floatx4_t w = {0.f, 0.f, 0.f, 0.f}, out = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+        for (int kt = 0; kt < KTW; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 w = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.kt[kt], r), S[kt][r], w, 0, 0, 0);
                 out = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.qt[kt], r), S[kt][r], out, 0, 0, 0);
             }
+        float (*mine)[2][4][WAVE] = shares[run & 1];
+        if constexpr (SW > 1) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                mine[wave][0][r][lane] = w[r];
+                mine[wave][1][r][lane] = out[r];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float sum = mine[0][0][r][lane];
+#pragma unroll
+                for (int j = 1; j < SW; ++j) sum += mine[j][0][r][lane];
+                w[r] = sum;
+            }
+        }
         w = cur.v - w;
         floatx4_t u = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < 4; ++r) u = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.tm, r), w[r], u, 0, 0, 0);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) out = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.p, r), u[r], out, 0, 0, 0);
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
+        for (int kt = 0; kt < KTW; ++kt) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[kt][r] *= at(cur.dec[kt], r);
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.kb[kt][r], u[r], S[kt], 0, 0, 0);
         }
-        if (live) {
+        // the read-out: P U on top of the shares of Qt S0; a wavefront stores the tokens 4 (lane / 16) + r with r its own
+        floatx4_t pu = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int tok = run * RUN + 4 * g4 + r;
-                if (tok < n) o[(static_cast<size_t>(first) + tok) * (H * dv) + h * dv + col] = out[r];
+        for (int r = 0; r < 4; ++r) pu = __builtin_amdgcn_mfma_f32_16x16x4f32(at(cur.p, r), u[r], pu, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (r % SW != wave) continue;
+            float val = pu[r];
+            if constexpr (SW > 1) {
+#pragma unroll
+                for (int j = 0; j < SW; ++j) val += mine[j][1][r][lane];
+            } else {
+                val += out[r];
             }
+            const int tok = run * RUN + 4 * g4 + r;
+            if (live && tok < n) o[(static_cast<size_t>(first) + tok) * (H * dv) + h * dv + col] = val;
         }
         cur = nxt;
     }
     if (live) {
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+        for (int kt = 0; kt < KTW; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) S_mem[kt * RUN + r] = S[kt][r];
     }
@@ -475,7 +509,7 @@ NI_EXPORT int ni_delta_rule(const void* prep, void* chunks, void* state, const v
             const int runs = (max_q_len + RUN - 1) / RUN;
             delta_chunk_prepare_kernel<<<dim3(B, runs, H), 256, 0, stream>>>((const float*)prep, (float*)chunks, (const int32_t*)q_start,
                                                                              (const int32_t*)q_len, G, H, dv);
-            delta_chunk_scan_kernel<<<dim3(B, H, (dv + RUN - 1) / RUN), 64, 0, stream>>>(
+            delta_chunk_scan_kernel<<<dim3(B, H, (dv + RUN - 1) / RUN), 64 * scan_waves(KPT * PARTS / RUN), 0, stream>>>(
                 (const float*)prep, (const float*)chunks, (float*)state, (const int32_t*)q_start, (const int32_t*)q_len,
                 (const int32_t*)state_slot, (float*)o, G, H, dv, state_stride);
         } else {
