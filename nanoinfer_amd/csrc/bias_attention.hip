@@ -244,6 +244,152 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
     }
 }
 
+// ------------------------------------------------------------------ prompt portions on the matrix cores, in float32
+// The same attention for tiles of up to 64 rows of (token, head), sixteen a wavefront, with both products on
+// v_mfma_f32_16x16x4_f32 (true 32-bit products and sums; keys, values and queries are widened to float32 when they
+// are staged).  Key and value sizes are multiples of 16.
+//
+//   S^T[key, row]  = K[key, :] . Q[row, :]    K rows as the first operand, Q rows as the second.  The k index of
+//                    an MFMA is only a label: lane group kg (lane / 16) of step t takes channel kg dk/4 + t, so
+//                    a lane reads dk/4 consecutive floats of its key and of its row.  A lane ends up with the
+//                    scores of ONE row (lane % 16) for keys 16 j + 4 kg + r: bias, temperature and the running
+//                    softmax are per lane, the row's maximum and sum cross the four lane groups only.
+//   O^T[dim, row] += V^T[dim, key] . P^T[key, row]   the weight of key 16 j + 4 kg + r is register (j, r) of the
+//                    lane, which is where the second operand of the MFMA over keys {16 j + 4 kg + r} wants it:
+//                    the weights never leave the registers.  The lane holds dims 16 db + 4 kg + r of its row.
+#define MROWS 64
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float groups4(float x, bool take_max) {
+    // over the four lanes that hold one row (lanes r, r + 16, r + 32, r + 48): maximum or sum
+    const auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    const float u = __uint_as_float(a[0]), v = __uint_as_float(a[1]);
+    x = take_max ? fmaxf(u, v) : u + v;
+    const auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    const float s = __uint_as_float(b[0]), t = __uint_as_float(b[1]);
+    return take_max ? fmaxf(s, t) : s + t;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(WAVES * WAVE)
+bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
+                           const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
+                           const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances,
+                           T* __restrict__ out, int H, int G, int dk, int dv, int page_size, float scale, float temp_coef,
+                           int temp_every, int heads_per_chunk, bool k_pieces, bool v_pieces) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int dkp = dk + 4, dvp = dv + 4;         // strides that spread the sixteen rows of a read over the banks
+    float* Qs = lds;                              // [MROWS][dkp]
+    float* Ks = Qs + MROWS * dkp;                 // [KEYS][dkp]
+    float* Vs = Ks + KEYS * dkp;                  // [KEYS][dvp]
+    const int tile = blockIdx.x, g = blockIdx.y, chunk = blockIdx.z;
+    const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2];
+    const int first_pos = positions[first_row];
+    const int group = H / G;
+    const int heads_here = std::min(heads_per_chunk, group - chunk * heads_per_chunk);
+    const int head0 = g * group + chunk * heads_per_chunk;
+    const int n_rows = n_tok * heads_here;        // row r = token r / heads_here, head r % heads_here
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int i = lane & 15, kg = lane >> 4;
+
+    for (int e = tid; e < MROWS * dk; e += blockDim.x) {
+        const int r = e / dk, c = e % dk;
+        float v = 0.f;
+        if (r < n_rows)
+            v = ld(qkv + static_cast<size_t>(first_row + r / heads_here) * row_stride + (head0 + r % heads_here) * dk + c);
+        Qs[r * dkp + c] = v;
+    }
+    const int row = wave * 16 + i;
+    const bool valid = row < n_rows;
+    const int pos = first_pos + (valid ? row / heads_here : 0);
+    const int head = head0 + (valid ? row % heads_here : 0);
+    const int steps = temp_every > 0 ? (pos + 1) / temp_every : 0;
+    const float factor = scale * (1.0f + temp_coef * logf(static_cast<float>(steps) + 1.0f));
+    // the last position any row of this wavefront has (the same for all its lanes)
+    const int wave_rows = std::min(16, n_rows - wave * 16);
+    const int wave_last = wave_rows > 0 ? first_pos + (wave * 16 + wave_rows - 1) / heads_here : -1;
+    float m = -INFINITY, l = 0.f;
+    floatx4_t acc[MAX_VCHUNKS * 4];               // dv / 16 blocks of [4 dims] of the lane's row
+#pragma unroll
+    for (int db = 0; db < MAX_VCHUNKS * 4; ++db) acc[db] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    const int dvb = dv / 16, qsteps = dk / 16;    // value blocks; 16-byte reads of a lane's quarter of a row
+    const int last_pos = first_pos + n_tok - 1;
+    const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
+    const float* qrow = Qs + row * dkp + kg * (dk / 4);
+    for (int k0 = 0; k0 <= last_pos; k0 += KEYS) {
+        __syncthreads();                          // the tile before this one has been used by everyone
+        stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, last_pos, k_pieces);
+        stage_rows<T>(vpool, Vs, dvp, dv, table, page_size, G, g, k0, last_pos, v_pieces);
+        __syncthreads();
+        if (k0 > wave_last) continue;             // nothing here for this wavefront's rows (it still stages and waits)
+        floatx4_t sc[KEYS / 16];
+#pragma unroll
+        for (int j = 0; j < KEYS / 16; ++j) sc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int t4 = 0; t4 < qsteps; ++t4) {
+            const float4 qv = *reinterpret_cast<const float4*>(qrow + 4 * t4);
+#pragma unroll
+            for (int j = 0; j < KEYS / 16; ++j) {
+                const float4 kv = *reinterpret_cast<const float4*>(Ks + (16 * j + i) * dkp + kg * (dk / 4) + 4 * t4);
+                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.x, qv.x, sc[j], 0, 0, 0);
+                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.y, qv.y, sc[j], 0, 0, 0);
+                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.z, qv.z, sc[j], 0, 0, 0);
+                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.w, qv.w, sc[j], 0, 0, 0);
+            }
+        }
+        float top = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < KEYS / 16; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = k0 + 16 * j + 4 * kg + r;
+                float v = -INFINITY;
+                if (valid && key <= pos) {
+                    const int back = std::min(pos - key, distances - 1);
+                    v = sc[j][r] * factor + (bias ? bias[static_cast<size_t>(back) * H + head] : 0.f);
+                }
+                sc[j][r] = v;
+                top = fmaxf(top, v);
+            }
+        top = groups4(top, true);
+        const float m_new = fmaxf(m, top);
+        const bool any = m_new > -INFINITY;       // a row that is no row, or whose keys all lie ahead, sees nothing
+        const float alpha = any ? expf(m - m_new) : 1.f;          // 0 at the row's first keys
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < KEYS / 16; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float p = any ? expf(sc[j][r] - m_new) : 0.f;           // e^-inf = 0 for a key that is not seen
+                sc[j][r] = p;
+                sum += p;
+            }
+        l = l * alpha + groups4(sum, false);
+        m = m_new;
+#pragma unroll
+        for (int db = 0; db < MAX_VCHUNKS * 4; ++db) {
+            if (db < dvb) {
+                floatx4_t a = acc[db] * alpha;
+#pragma unroll
+                for (int j = 0; j < KEYS / 16; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        a = __builtin_amdgcn_mfma_f32_16x16x4f32(Vs[(16 * j + 4 * kg + r) * dvp + 16 * db + i], sc[j][r], a, 0, 0, 0);
+                acc[db] = a;
+            }
+        }
+    }
+    if (!valid) return;
+    T* orow = out + static_cast<size_t>(first_row + row / heads_here) * (H * dv) + head * dv + 4 * kg;
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int db = 0; db < MAX_VCHUNKS * 4; ++db) {
+        if (db < dvb) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) st(orow + 16 * db + r, acc[db][r] * inv);
+        }
+    }
+}
+
 // out[row, :] = sum_r acc_r e^(m_r - M) / sum_r l_r e^(m_r - M) over the runs of a row (an empty run has l = 0)
 template <typename T>
 __global__ void merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv) {
@@ -316,6 +462,49 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
             temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp);
         if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv);
+    }
+    return NI_LAUNCH_RESULT();
+}
+
+// rows of (token, head) of a tile of the matrix-core kernel; 0 where it does not take these sizes
+NI_EXPORT int ni_bias_attention_mfma_rows(int dk, int dv) {
+    if (dk % 16 || dv % 16 || dk < 16 || dv < 16 || dv > MAX_VCHUNKS * WAVE) return 0;
+    const size_t lds = (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + static_cast<size_t>(KEYS) * (dv + 4)) * sizeof(float);
+    return lds <= 160 * 1024 ? MROWS : 0;
+}
+
+// tiles of up to 64 rows (tokens * heads of a chunk), no runs: for steps with portions of prompts
+NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
+                                     int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias,
+                                     int distances, void* out, int H, int G, int dk, int dv, int page_size, float scale,
+                                     float temp_coef, int temp_every, int heads_per_chunk, int dtype, hipStream_t stream) {
+    if (n_tiles <= 0) return 0;
+    if (!ni_bias_attention_mfma_rows(dk, dv) || H % G || heads_per_chunk < 1 || heads_per_chunk > MROWS) return -1;
+    const int group = H / G;
+    const size_t lds = (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + static_cast<size_t>(KEYS) * (dv + 4)) * sizeof(float);
+    const int vec = dtype == 0 ? 4 : 8;
+    const bool k_pieces = dk % vec == 0 && reinterpret_cast<uintptr_t>(kpool) % 16 == 0;
+    const bool v_pieces = dv % vec == 0 && reinterpret_cast<uintptr_t>(vpool) % 16 == 0;
+    dim3 grid(n_tiles, G, (group + heads_per_chunk - 1) / heads_per_chunk);
+    hipError_t err = hipSuccess;
+    if (dtype == 0) {
+        static size_t allowed = 48 * 1024;
+        if (lds > allowed && (allowed = lds))
+            err = hipFuncSetAttribute((const void*)bias_attention_mfma_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return (int)err;
+        bias_attention_mfma_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
+            (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
+            (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size,
+            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces);
+    } else {
+        static size_t allowed = 48 * 1024;
+        if (lds > allowed && (allowed = lds))
+            err = hipFuncSetAttribute((const void*)bias_attention_mfma_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return (int)err;
+        bias_attention_mfma_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
+            (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
+            (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size,
+            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces);
     }
     return NI_LAUNCH_RESULT();
 }

@@ -1184,6 +1184,6 @@ torch.backends.cuda.matmul.allow_tf32 = False
 torch.backends.cudnn.allow_tf32 = False
 
 # sums onto the residual stream, routed experts, the gated delta rule, attention with a bias by distance
-from .stream import (EXPERTS_FEW_ROWS, add_rmsnormed, add_vector, bias_attention, bias_attention_lib,  # noqa: E402,F401
-                     bias_attention_rows, bias_attention_runs, delta_rule, delta_rule_lib, embed_scaled, experts_act, experts_few,
+from .stream import (BIAS_ATTENTION_MFMA_FROM, DELTA_RUN_FROM, EXPERTS_FEW_ROWS, add_rmsnormed, add_vector,  # noqa: E402,F401
+                     bias_attention, bias_attention_lib, bias_attention_mfma, bias_attention_mfma_rows, bias_attention_rows, bias_attention_runs, delta_rule, delta_rule_lib, embed_scaled, experts_act, experts_few,
                      gated_side, kv_store, route_top, stream_add, stream_lib)

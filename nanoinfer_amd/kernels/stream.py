@@ -285,3 +285,45 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
         raise KernelError(f"keys of {dk} and values of {dv} channels do not fit the kernel's staging memory")
     _check(err, "bias_attention")
     return out
+
+
+BIAS_ATTENTION_MFMA_FROM = 8      # a step whose longest portion has this many tokens takes the matrix-core kernel
+
+
+def bias_attention_mfma_rows(dk: int, dv: int) -> int:
+    """Rows of (token, head) of a tile of the matrix-core kernel for prompt portions; 0 where it does not take
+    these sizes (both multiples of 16, small enough for its staging memory)."""
+    return int(bias_attention_lib().ni_bias_attention_mfma_rows(int(dk), int(dv)))
+
+
+def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                        tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int,
+                        scale: float, temp_coef: float, temp_every: int, heads_per_chunk: int) -> torch.Tensor:
+    """:func:`bias_attention` for steps with portions of prompts: tiles of up to 64 rows (tokens * heads of a chunk),
+    both products on the float32 matrix instructions, the same formula and the same 32-bit softmax; no runs."""
+    T, width = qkv.shape
+    pages, G, ps, dk = kpool.shape
+    dv = vpool.shape[3]
+    _gpu(qkv, "qkv")
+    _gpu(kpool, "kpool", qkv.dtype)
+    _gpu(vpool, "vpool", qkv.dtype, (pages, G, ps, dv))
+    _need(block_table.is_cuda and block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be int32 [B, pages] on the GPU")
+    _need(tiles.is_cuda and tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
+          "tiles must be int32 [n, 4] on the GPU")
+    _gpu(out, "out", qkv.dtype, (T, H * dv))
+    _gpu(positions, "positions", torch.int32, (T,))
+    _need(H % G == 0 and H * dk <= width, "heads")
+    _need(bias_attention_mfma_rows(dk, dv) > 0, f"keys of {dk} and values of {dv} channels are not taken by the matrix-core kernel")
+    _need(1 <= heads_per_chunk <= 64, "heads_per_chunk")
+    distances = 0
+    if bias is not None:
+        distances = bias.shape[0]
+        _gpu(bias, "bias", torch.float32, (distances, H))
+        _need(distances >= 1, "an empty bias table")
+    _check(bias_attention_lib().ni_bias_attention_mfma(_ptr(qkv), width, _ptr(kpool), _ptr(vpool), _ptr(block_table),
+                                                       block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions),
+                                                       _ptr(bias), distances, _ptr(out), H, G, dk, dv, ps, _float(scale),
+                                                       _float(temp_coef), int(temp_every), heads_per_chunk,
+                                                       dtype_code(qkv.dtype), _stream()), "bias_attention_mfma")
+    return out

@@ -197,6 +197,10 @@ class BiasAttention(Part):
         self.heads_per_chunk = min(group, K.bias_attention_rows())
         self.tile_tokens = max(1, K.bias_attention_rows() // self.heads_per_chunk)
         K.bias_attention_lib()
+        # steps with portions of prompts: larger tiles on the matrix cores, where the kernel takes these sizes
+        wide = K.bias_attention_mfma_rows(self.dk, self.dv)
+        self.wide_heads = min(group, wide) if wide else 0
+        self.wide_tokens = max(1, wide // self.wide_heads) if wide else 0
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.G, self.dk, None, self.dv))
@@ -206,10 +210,17 @@ class BiasAttention(Part):
         qkv = K.linear(x, self.w_qkv)
         if cache.writes:
             K.kv_store(qkv, self.H * self.dk, (self.H + self.G) * self.dk, cache.slot_mapping, cache.kpool, cache.vpool)
+        out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
+        if self.wide_heads and ctx.max_q_len >= K.BIAS_ATTENTION_MFMA_FROM:
+            tiles = ctx.q_tiles(self.wide_tokens)
+            if tiles is None:
+                raise K.KernelError("this step was recorded without the tiles of its tokens")
+            K.bias_attention_mfma(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H,
+                                  self.scale, self.temp_coef, self.temp_every, self.wide_heads)
+            return K.linear(out, self.w_o, out_dtype=torch.float32)
         tiles = ctx.q_tiles(self.tile_tokens)
         if tiles is None:
             raise K.KernelError("this step was recorded without the tiles of its tokens")
-        out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
         chunks = -(-(self.H // self.G) // self.heads_per_chunk)
         # a step of single tokens has tiles of one token: its rows are the heads of a chunk, four a wavefront
         rows = min(self.tile_tokens, ctx.max_q_len) * self.heads_per_chunk

@@ -335,6 +335,91 @@ def test_few_rows_and_many_rows_of_routed_experts_agree_with_the_plain_sum(dtype
         assert err < tol, (name, err)
 
 
+# ------------------------------------------------------------------ the attention's two kernels
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,dk,dv,page,bias_rows,temp", [(8, 1, 64, 80, 16, 12, (0.3, 8)), (6, 2, 16, 16, 4, None, None),
+                                                          (20, 1, 32, 48, 8, 6, None), (3, 3, 48, 16, 32, None, (0.5, 3))])
+def test_attention_on_the_matrix_cores_and_on_the_vector_units_agree_with_the_plain_softmax(H, G, dk, dv, page, bias_rows, temp, dtype):
+    """Three sequences in one step: a portion of 70 tokens after 150 cached ones (keys far back, tiles that end
+    inside a portion), a whole prompt of 9 and a single token after 64, on pages handed out in a scattered order.
+    Both kernels against the softmax written out in float64 on the same (rounded) q, k, v."""
+    from nanoinfer_amd import kernels as K
+    from nanoinfer_amd.parts.hybrid import distance_rows
+    g = torch.Generator().manual_seed(H * dk + dv)
+    dev = torch.device("cuda")
+    ctx_before, q_len = [150, 0, 64], [70, 9, 1]
+    total = [a + b for a, b in zip(ctx_before, q_len)]
+    T = sum(q_len)
+    q_start = [sum(q_len[:i]) for i in range(3)]
+    pages_per = [-(-t // page) for t in total]
+    n_pages = sum(pages_per) + 3
+    order = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.full((3, max(pages_per) + 1), -1, dtype=torch.int32)
+    kpool = torch.full((n_pages, G, page, dk), float("nan"))
+    vpool = torch.full((n_pages, G, page, dv), float("nan"))
+    keys, values = [], []
+    for s in range(3):
+        k = (torch.randn(total[s], G, dk, generator=g) * 0.8).to(dtype).float()
+        v = torch.randn(total[s], G, dv, generator=g).to(dtype).float()
+        k[3] *= 4.0                                  # one key far back that many queries look at
+        keys.append(k); values.append(v)
+        for j in range(pages_per[s]):
+            pg = order.pop()
+            table[s, j] = pg
+            n = min(page, total[s] - j * page)
+            kpool[pg, :, :n] = k[j * page: j * page + n].transpose(0, 1)
+            vpool[pg, :, :n] = v[j * page: j * page + n].transpose(0, 1)
+            kpool[pg, :, n:] = 0.0                   # slots of the page that no token has yet hold whatever: finite here
+            vpool[pg, :, n:] = 0.0
+    kpool, vpool = torch.nan_to_num(kpool, nan=1e30), torch.nan_to_num(vpool, nan=1e30)     # pages of nobody: huge
+    q = (torch.randn(T, H, dk, generator=g) * 0.8).to(dtype).float()
+    positions = [ctx_before[s] + i for s in range(3) for i in range(q_len[s])]
+    scale = 0.21
+    bias = None
+    if bias_rows is not None:
+        learned = torch.randn(bias_rows, H, generator=g) * 2.0
+        bias = learned[torch.from_numpy(distance_rows(bias_rows, 100.0, 256))].contiguous()
+    want = torch.zeros(T, H, dv, dtype=torch.float64)
+    for s in range(3):
+        for i in range(q_len[s]):
+            row, p = q_start[s] + i, ctx_before[s] + i
+            f = scale * (1.0 if temp is None else 1.0 + temp[0] * __import__("math").log((p + 1) // temp[1] + 1))
+            for h in range(H):
+                kv = h // (H // G)
+                sc = (keys[s][: p + 1, kv].double() @ q[row, h].double()) * f
+                if bias is not None:
+                    sc = sc + bias[[p - j for j in range(p + 1)], h].double()
+                want[row, h] = torch.softmax(sc, dim=0) @ values[s][: p + 1, kv].double()
+    qkv = torch.zeros(T, H * dk + 5, dtype=dtype)
+    qkv[:, : H * dk] = q.reshape(T, H * dk).to(dtype)
+    qkv, kp, vp = qkv.to(dev), kpool.to(dev, dtype), vpool.to(dev, dtype)
+    pos_d = torch.tensor(positions, dtype=torch.int32, device=dev)
+    bias_d = None if bias is None else bias.to(dev)
+    tc, te = (0.0, 0) if temp is None else temp
+    group = H // G
+
+    def tiles(tokens):
+        flat = K.build_q_tiles(q_start, q_len, total, tokens)
+        return torch.tensor(flat, dtype=torch.int32, device=dev).view(-1, 4)
+
+    results = {}
+    hpc = min(group, K.bias_attention_rows())
+    out = torch.empty(T, H * dv, dtype=dtype, device=dev)
+    K.bias_attention(qkv, kp, vp, table.to(dev), tiles(max(1, K.bias_attention_rows() // hpc)), pos_d, bias_d, out, H, scale, tc, te, hpc)
+    results["vector units"] = out
+    wide = K.bias_attention_mfma_rows(dk, dv)
+    assert wide == 64
+    hpc = min(group, wide)
+    out = torch.empty(T, H * dv, dtype=dtype, device=dev)
+    K.bias_attention_mfma(qkv, kp, vp, table.to(dev), tiles(max(1, wide // hpc)), pos_d, bias_d, out, H, scale, tc, te, hpc)
+    results["matrix cores"] = out
+    tol = 2e-5 if dtype == torch.float32 else 6e-3          # bfloat16: the rounding of the output alone
+    for name, got in results.items():
+        err = float((got.double().cpu().view(T, H, dv) - want).abs().max() / want.abs().max())
+        assert err < tol, (name, err)
+
+
 # ------------------------------------------------------------------ the delta rule's two kernels
 
 def _plain_delta_step(proj, low, conv, a_log, dt_bias, norm_w, state, starts, lens, slots, G, H, dk, dv, taps, eps):
