@@ -381,20 +381,23 @@ def serving(args) -> int:
 
 
 # ---------------------------------------------------------------- --workload hybrid
-# A Zekalorn model whose layers have the sizes of the 1B shape's (width 2,048, feed-forwards of 8,192 or sixteen
-# experts of 1,024 of which a token uses four, attention of 32 heads on 8 of size 64, delta-rule layers of 16
-# heads with keys and values of 128), beside the Llama shape of as many layers and the same vocabulary.
+# A Zekalorn model whose layers have the sizes of a Llama shape's (--shape: its width, feed-forwards of its size or
+# sixteen experts of an eighth of it of which a token uses four, attention with its heads and head size, delta-rule
+# layers of width / 128 heads with keys and values of 128), beside that Llama shape with as many layers and the
+# same vocabulary.
 
-def hybrid_config(layers: int, vocab: int, positions: int) -> dict:
-    delta = {"type": "channel_delta", "mixer": {"heads": 16, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4,
+def hybrid_config(layers: int, vocab: int, positions: int, like: dict) -> dict:
+    width, ff = like["hidden_size"], like["intermediate_size"]
+    delta = {"type": "channel_delta", "mixer": {"heads": width // 128, "kv_heads": width // 128, "dim": 128, "vdim": 128, "conv": 4,
                                                 "decay_rank": 64, "gate_rank": 64}}
-    attn = {"type": "attention", "mixer": {"heads": 32, "kv_heads": 8, "dim": 64, "vdim": 64, "scale": 0.125, "bias_max": 4096.0,
-                                           "bias_rows": 64, "q_temp": {"coef": 0.1, "every": 1024}}}
-    dense = {"kind": "dense", "ff": 8192}
-    routed = {"kind": "moe", "expert": {"ff": 1024}, "router": {"experts": 16, "top": 4}}
+    attn = {"type": "attention", "mixer": {"heads": like["num_attention_heads"], "kv_heads": like["num_key_value_heads"],
+                                           "dim": like["head_dim"], "vdim": like["head_dim"], "scale": like["head_dim"] ** -0.5,
+                                           "bias_max": 4096.0, "bias_rows": 64, "q_temp": {"coef": 0.1, "every": 1024}}}
+    dense = {"kind": "dense", "ff": ff}
+    routed = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 16, "top": 4}}
     pattern = [(delta, dense), (delta, routed), (delta, dense), (attn, routed)]
-    return {"architecture": "Zekalorn", "vocab": vocab, "width": 2048, "max_positions": positions,
-            "embedding": {"scale": 45.25}, "norm": {"eps": 1e-5}, "token_side": {"dim": 64},
+    return {"architecture": "Zekalorn", "vocab": vocab, "width": width, "max_positions": positions,
+            "embedding": {"scale": float(width) ** 0.5}, "norm": {"eps": 1e-5}, "token_side": {"dim": 64},
             "layers": [dict(pattern[i % 4][0], mlp=pattern[i % 4][1]) for i in range(layers)]}
 
 
@@ -407,9 +410,11 @@ def hybrid(args) -> int:
     prompt, batch = args.prompt_len, args.batch
     out = {"metric": "hybrid_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
-           "config": {"layers": layers, "prompt_len": prompt, "global_batch": batch, "width": 2048, "vocab": 128256}}
-    shapes = {"zekalorn": hybrid_config(layers, 128256, prompt + 2048),
-              "llama": dict(LLAMA_1B, num_hidden_layers=layers, max_position_embeddings=prompt + 2048)}
+           "config": {"layers": layers, "prompt_len": prompt, "global_batch": batch, "shape": args.shape,
+                      "width": SHAPES[args.shape][2]["hidden_size"], "vocab": 128256}}
+    like = SHAPES[args.shape][2]
+    shapes = {"zekalorn": hybrid_config(layers, 128256, prompt + 2048, like),
+              "llama": dict(like, num_hidden_layers=layers, max_position_embeddings=prompt + 2048)}
     for name, cfg in shapes.items():
         if args.only and name != args.only:
             continue

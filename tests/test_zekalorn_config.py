@@ -137,3 +137,18 @@ def test_plain_routing_with_all_experts_chosen_is_a_full_softmax():
     mix = torch.softmax(P.linear(n, w["router"]), dim=-1)
     want = sum(mix[:, e:e + 1] * P.linear(torch.relu(P.linear(n, w[f"e{e}.up"])) ** 2, w[f"e{e}.down"]) for e in range(E))
     assert torch.allclose(P.routed_ff(n, w, E, E), want)
+
+
+@pytest.mark.parametrize("shape", ["1b", "3b", "8b"])
+def test_the_bench_shapes_are_valid_configurations(shape):
+    """``bench.py --workload hybrid --shape ...`` writes a Zekalorn model with the layer sizes of that Llama shape."""
+    import bench
+    like = bench.SHAPES[shape][2]
+    d = bench.hybrid_config(8, 1000, 4096, like)
+    cfg = ZekalornConfig.from_dict(d)
+    spec = architecture_of(d).build_spec(cfg)
+    assert len(spec.order) == 8
+    mixers = [layer["type"] for layer in d["layers"]]
+    assert mixers.count("attention") == 2 and mixers.count("channel_delta") == 6
+    attn = next(layer["mixer"] for layer in d["layers"] if layer["type"] == "attention")
+    assert attn["heads"] == like["num_attention_heads"] and attn["dim"] == like["head_dim"]
