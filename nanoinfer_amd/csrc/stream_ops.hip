@@ -240,87 +240,127 @@ NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int
 // take neighbouring pieces of the row, so a row streams from memory in whole lines.
 //   hid[t * top + k, i] = relu(W_up[chosen[t, k] * ff + i, :] . x[t, :])^2        (float32)
 //   out[t, r] = sum_k mix[t, k] * W_down[r, chosen[t, k] * ff : +ff] . hid[t * top + k, :]
-template <typename T>
+// A wavefront takes R neighbouring rows at once, with a sum of its own for each: the loads of the R rows are in
+// flight together, and the input row is read once for all of them.
+template <typename T, int R>
 __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restrict__ w_up, const int32_t* __restrict__ chosen,
-                                      float* __restrict__ hid, int d, int ff, int top, int rows_per_block, bool vec) {
+                                      float* __restrict__ hid, int d, int ff, int top, bool vec) {
     const int pair = blockIdx.x;                 // t * top + k
     const int t = pair / top;
     const int e = chosen[pair];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
     const T* xr = x + static_cast<size_t>(t) * d;
-    const int first = blockIdx.y * rows_per_block;
-    for (int i = first + wave; i < first + rows_per_block && i < ff; i += waves) {
-        const T* wr = w_up + (static_cast<size_t>(e) * ff + i) * d;
-        float s = 0.f;
-        if (vec) {          // eight elements a lane and load: a wavefront takes 512 neighbouring elements at once
-            for (int c = lane * 8; c < d; c += WAVE * 8) {
-                float wv[8], xv[8];
-                VecIO<T, 8>::load(wr + c, wv);
-                VecIO<T, 8>::load(xr + c, xv);
+    const int i0 = (blockIdx.y * waves + wave) * R;
+    if (i0 >= ff) return;
+    const T* wr[R];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) s += wv[j] * xv[j];
-            }
-        } else {
-            for (int c = lane; c < d; c += WAVE) s += ld(wr + c) * ld(xr + c);
+    for (int u = 0; u < R; ++u) wr[u] = w_up + (static_cast<size_t>(e) * ff + min(i0 + u, ff - 1)) * d;
+    float s[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) s[u] = 0.f;
+    if (vec) {          // eight elements a lane and load: a wavefront takes 512 neighbouring elements of a row at once
+        for (int c = lane * 8; c < d; c += WAVE * 8) {
+            float wv[R][8], xv[8];
+#pragma unroll
+            for (int u = 0; u < R; ++u) VecIO<T, 8>::load(wr[u] + c, wv[u]);
+            VecIO<T, 8>::load(xr + c, xv);
+#pragma unroll
+            for (int u = 0; u < R; ++u)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) s[u] += wv[u][j] * xv[j];
         }
-        s = wave_sum(s);
-        if (lane == 0) {
-            const float u = fmaxf(s, 0.f);
-            hid[static_cast<size_t>(pair) * ff + i] = u * u;
+    } else {
+        for (int c = lane; c < d; c += WAVE) {
+            const float xv = ld(xr + c);
+#pragma unroll
+            for (int u = 0; u < R; ++u) s[u] += ld(wr[u] + c) * xv;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const float v = wave_sum(s[u]);
+        if (lane == 0 && i0 + u < ff) {
+            const float a = fmaxf(v, 0.f);
+            hid[static_cast<size_t>(pair) * ff + i0 + u] = a * a;
         }
     }
 }
 
-template <typename T>
+template <typename T, int R>
 __global__ void experts_down_few_kernel(const float* __restrict__ hid, const T* __restrict__ w_down,
                                         const int32_t* __restrict__ chosen, const float* __restrict__ mix,
-                                        float* __restrict__ out, int d, int ff, int E, int top, int rows_per_block, bool vec) {
+                                        float* __restrict__ out, int d, int ff, int E, int top, bool vec) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
-    const int first = blockIdx.y * rows_per_block;
+    const int r0 = (blockIdx.y * waves + wave) * R;
+    if (r0 >= d) return;
     const size_t row_stride = static_cast<size_t>(E) * ff;
-    for (int r = first + wave; r < first + rows_per_block && r < d; r += waves) {
-        float total = 0.f;
-        for (int k = 0; k < top; ++k) {
-            const int e = chosen[t * top + k];
-            const T* wr = w_down + static_cast<size_t>(r) * row_stride + static_cast<size_t>(e) * ff;
-            const float* hr = hid + (static_cast<size_t>(t) * top + k) * ff;
-            float s = 0.f;
-            if (vec) {
-                for (int c = lane * 8; c < ff; c += WAVE * 8) {
-                    float wv[8], hv[8];
-                    VecIO<T, 8>::load(wr + c, wv);
-                    VecIO<float, 8>::load(hr + c, hv);
+    float total[R];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) s += wv[j] * hv[j];
-                }
-            } else {
-                for (int c = lane; c < ff; c += WAVE) s += ld(wr + c) * hr[c];
+    for (int u = 0; u < R; ++u) total[u] = 0.f;
+    for (int k = 0; k < top; ++k) {
+        const int e = chosen[t * top + k];
+        const float* hr = hid + (static_cast<size_t>(t) * top + k) * ff;
+        const T* wr[R];
+#pragma unroll
+        for (int u = 0; u < R; ++u) wr[u] = w_down + static_cast<size_t>(min(r0 + u, d - 1)) * row_stride + static_cast<size_t>(e) * ff;
+        float s[R];
+#pragma unroll
+        for (int u = 0; u < R; ++u) s[u] = 0.f;
+        if (vec) {
+            for (int c = lane * 8; c < ff; c += WAVE * 8) {
+                float wv[R][8], hv[8];
+#pragma unroll
+                for (int u = 0; u < R; ++u) VecIO<T, 8>::load(wr[u] + c, wv[u]);
+                VecIO<float, 8>::load(hr + c, hv);
+#pragma unroll
+                for (int u = 0; u < R; ++u)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) s[u] += wv[u][j] * hv[j];
             }
-            total += mix[t * top + k] * wave_sum(s);
+        } else {
+            for (int c = lane; c < ff; c += WAVE) {
+                const float hv = hr[c];
+#pragma unroll
+                for (int u = 0; u < R; ++u) s[u] += ld(wr[u] + c) * hv;
+            }
         }
-        if (lane == 0) out[static_cast<size_t>(t) * d + r] = total;
+        const float weight = mix[t * top + k];
+#pragma unroll
+        for (int u = 0; u < R; ++u) total[u] += weight * wave_sum(s[u]);
     }
+    if (lane == 0) {
+#pragma unroll
+        for (int u = 0; u < R; ++u)
+            if (r0 + u < d) out[static_cast<size_t>(t) * d + r0 + u] = total[u];
+    }
+}
+
+template <typename T, int R>
+static void launch_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
+                               void* hid, void* out, int T_, int d, int ff, int E, int top, bool vec_up, bool vec_down,
+                               hipStream_t stream) {
+    constexpr int rows = 4 * R;                  // four wavefronts a workgroup
+    dim3 g1(T_ * top, (ff + rows - 1) / rows), g2(T_, (d + rows - 1) / rows);
+    experts_up_few_kernel<T, R><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up);
+    experts_down_few_kernel<T, R><<<g2, 256, 0, stream>>>((const float*)hid, (const T*)w_down, (const int32_t*)chosen,
+                                                          (const float*)mix, (float*)out, d, ff, E, top, vec_down);
 }
 
 NI_EXPORT int ni_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
                              void* hid, void* out, int T, int d, int ff, int E, int top, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
-    const int rows = 16;
-    dim3 g1(T * top, (ff + rows - 1) / rows), g2(T, (d + rows - 1) / rows);
     // rows of whole 16-byte (bfloat16) or 32-byte (float32) pieces that start on such a piece are read in pieces
     const bool vec_up = d % 8 == 0 && aligned16(x, w_up);
     const bool vec_down = ff % 8 == 0 && aligned16(w_down, hid);
+    // four rows a wavefront where that still leaves the second kernel a workgroup for every compute unit, else two
+    const bool four = static_cast<long long>(T) * ((d + 15) / 16) >= 256;
     if (dtype == 0) {
-        experts_up_few_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)w_up, (const int32_t*)chosen,
-                                                             (float*)hid, d, ff, top, rows, vec_up);
-        experts_down_few_kernel<float><<<g2, 256, 0, stream>>>((const float*)hid, (const float*)w_down, (const int32_t*)chosen,
-                                                               (const float*)mix, (float*)out, d, ff, E, top, rows, vec_down);
+        if (four) launch_experts_few<float, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
+        else launch_experts_few<float, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
     } else {
-        experts_up_few_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w_up, (const int32_t*)chosen,
-                                                              (float*)hid, d, ff, top, rows, vec_up);
-        experts_down_few_kernel<bf16_t><<<g2, 256, 0, stream>>>((const float*)hid, (const bf16_t*)w_down, (const int32_t*)chosen,
-                                                                (const float*)mix, (float*)out, d, ff, E, top, rows, vec_down);
+        if (four) launch_experts_few<bf16_t, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
+        else launch_experts_few<bf16_t, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
     }
     return NI_LAUNCH_RESULT();
 }
