@@ -68,19 +68,25 @@ __device__ __forceinline__ float conv_at(const float* __restrict__ proj, const f
 
 __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float* __restrict__ low,
                                      const float* __restrict__ conv, const float* __restrict__ a_log,
-                                     const float* __restrict__ dt_bias, const float* __restrict__ state,
+                                     const float* __restrict__ dt_bias, float* __restrict__ state,
                                      const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
                                      const int32_t* __restrict__ state_slot, float* __restrict__ prep,
                                      int G, int H, int dk, int dv, int taps, int proj_cols, size_t state_stride,
-                                     size_t conv_off, int log_decay) {
+                                     size_t conv_off, int log_decay, int move_on) {
     __shared__ float scratch[16];
     const int t = blockIdx.x, unit = blockIdx.y;
     const int s = seq_of_token[t];
     const int i = t - q_start[s];              // place of the token in its portion
     const int QK = 2 * G * dk, C = QK + H * dv;
     const int prep_cols = C + H + H * dk + H * dv;
-    const float* hist = state + static_cast<size_t>(state_slot[s]) * state_stride + conv_off;
+    float* hist = state + static_cast<size_t>(state_slot[s]) * state_stride + conv_off;
     float* out = prep + static_cast<size_t>(t) * prep_cols;
+    // move_on: every sequence of the step brings one token, so the thread that has read a channel's last inputs is the
+    // only one that does, and moves them on itself (no kernel of its own for that)
+    auto moved = [&](int c) {
+        for (int j = 0; j + 2 < taps; ++j) hist[static_cast<size_t>(j) * C + c] = hist[static_cast<size_t>(j + 1) * C + c];
+        hist[static_cast<size_t>(taps - 2) * C + c] = proj[static_cast<size_t>(t) * proj_cols + c];
+    };
     if (unit < 2 * G) {
         // a head of q or of k: every thread keeps its channels (dk <= 256 = threads)
         const int c = unit * dk + threadIdx.x;
@@ -88,6 +94,7 @@ __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float
         if (threadIdx.x < dk) {
             const float z = conv_at(proj, hist, conv, t, i, c, C, taps, proj_cols);
             y = z * (1.0f / (1.0f + expf(-z)));
+            if (move_on && taps > 1) moved(c);
         }
         const float ss = block_sum(y * y, scratch);
         const float inv = (1.0f / sqrtf(ss + 1e-6f)) * (unit < G ? 1.0f / sqrtf(static_cast<float>(dk)) : 1.0f);
@@ -101,6 +108,7 @@ __global__ void delta_prepare_kernel(const float* __restrict__ proj, const float
         const int c = QK + h * dv + j;
         const float z = conv_at(proj, hist, conv, t, i, c, C, taps, proj_cols);
         out[c] = z * (1.0f / (1.0f + expf(-z)));
+        if (move_on && taps > 1) moved(c);
         out[C + H + H * dk + h * dv + j] = 1.0f / (1.0f + expf(-lrow[H * dk + h * dv + j]));
     }
     const float rate = expf(a_log[h]);
@@ -472,18 +480,19 @@ NI_EXPORT int ni_delta_key_size() { return KPT * PARTS; }
 NI_EXPORT int ni_delta_prepare(const void* proj, const void* low, const void* conv, const void* a_log, const void* dt_bias,
                                void* state, const void* seq_of_token, const void* q_start, const void* q_len,
                                const void* state_slot, void* prep, int T, int B, int G, int H, int dk, int dv, int taps,
-                               int proj_cols, size_t state_stride, size_t conv_off, int log_decay, hipStream_t stream) {
+                               int proj_cols, size_t state_stride, size_t conv_off, int log_decay, int max_q_len, hipStream_t stream) {
     if (T <= 0) return 0;
+    const int move_on = max_q_len == 1;         // a step of single tokens: the prepare kernel moves the convolutions' inputs on
     if (dk != KPT * PARTS) return -1;
     const int C = 2 * G * dk + H * dv;
     if (dk > 256) return -2;
     const int widest = std::max(dk, std::min(dv, 256));
     delta_prepare_kernel<<<dim3(T, 2 * G + H), (widest + 63) / 64 * 64, 0, stream>>>((const float*)proj, (const float*)low, (const float*)conv,
-                                                  (const float*)a_log, (const float*)dt_bias, (const float*)state,
+                                                  (const float*)a_log, (const float*)dt_bias, (float*)state,
                                                   (const int32_t*)seq_of_token, (const int32_t*)q_start,
                                                   (const int32_t*)state_slot, (float*)prep, G, H, dk, dv, taps, proj_cols,
-                                                  state_stride, conv_off, log_decay);
-    if (taps > 1) {
+                                                  state_stride, conv_off, log_decay, move_on);
+    if (taps > 1 && !move_on) {
         dim3 grid(B, std::max(1, std::min(64, (C + 255) / 256)));
         conv_state_update_kernel<<<grid, 256, 0, stream>>>((const float*)proj, (float*)state, (const int32_t*)q_start,
                                                            (const int32_t*)q_len, (const int32_t*)state_slot, C, taps,

@@ -157,7 +157,7 @@ DELTA_RUN_FROM = 16      # a step whose longest portion has this many tokens goe
 def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                norm_w: torch.Tensor, state: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor,
                q_len: torch.Tensor, state_slot: torch.Tensor, G: int, H: int, dk: int, dv: int, taps: int, eps: float,
-               out_dtype: torch.dtype, max_q_len: int = 1) -> torch.Tensor:
+               out_dtype: torch.dtype, max_q_len: int = 0, runs: Optional[bool] = None) -> torch.Tensor:
     """One step of the gated delta rule with a decay per key channel for all sequences of the step.
 
     ``proj`` float32 [T, >= C + H] holds q [G*dk] | k [G*dk] | v [H*dv] | b [H] as projected (C the first
@@ -166,9 +166,11 @@ def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log:
     [head, value channel, key channel]) and the convolutions' last inputs, both moved on by this call.
     Returns the normalised, gated read-out [T, H*dv] in ``out_dtype``.
 
-    ``max_q_len`` is the longest portion of the step (a host number).  From ``DELTA_RUN_FROM`` tokens on, and
-    where the key size is a multiple of 16, the step goes sixteen tokens at a time on the matrix cores (in
-    float32 as well); otherwise token by token.  Both compute the same recurrence and differ by rounding."""
+    ``max_q_len`` is the longest portion of the step (a host number; 0: not known).  From ``DELTA_RUN_FROM``
+    tokens on, and where the key size is a multiple of 16, the step goes sixteen tokens at a time on the matrix
+    cores (in float32 as well); otherwise token by token (``runs`` = True / False asks for one of the two).
+    Both compute the same recurrence and differ by rounding.  A step of single tokens (``max_q_len`` 1) moves
+    the convolutions' inputs on in its first kernel."""
     T, proj_cols = proj.shape
     B = q_start.shape[0]
     C = 2 * G * dk + H * dv
@@ -189,14 +191,18 @@ def delta_rule(proj: torch.Tensor, low: torch.Tensor, conv: torch.Tensor, a_log:
     lib = delta_rule_lib(dk)
     prep = torch.empty(T, C + H + H * dk + H * dv, dtype=torch.float32, device=proj.device)
     stride = state.shape[1]
-    run_floats = int(lib.ni_delta_run_floats()) if max_q_len >= DELTA_RUN_FROM else 0
+    _need(0 <= max_q_len <= T, "max_q_len is larger than the step")
+    _need(max_q_len != 1 or T == B, "a step of single tokens has one row a sequence")
+    in_runs = max_q_len >= DELTA_RUN_FROM if runs is None else bool(runs)
+    run_floats = int(lib.ni_delta_run_floats()) if in_runs else 0
+    _need(run_floats > 0 or not runs, f"the delta rule has no runs of sixteen for keys of {dk} channels")
     chunks = None
     if run_floats:
-        _need(max_q_len <= T, "max_q_len is larger than the step")
+        max_q_len = max_q_len or T
         chunks = torch.empty((T // 16 + B + 1) * H * run_floats, dtype=torch.float32, device=proj.device)
     _check(lib.ni_delta_prepare(_ptr(proj), _ptr(low), _ptr(conv), _ptr(a_log), _ptr(dt_bias), _ptr(state), _ptr(seq_of_token),
                                 _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(prep), T, B, G, H, dk, dv, taps, proj_cols,
-                                _size_t(stride), _size_t(conv_off), int(chunks is not None), _stream()), "delta_prepare")
+                                _size_t(stride), _size_t(conv_off), int(chunks is not None), int(max_q_len), _stream()), "delta_prepare")
     o = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
     y = torch.empty(T, H * dv, dtype=out_dtype, device=proj.device)
     _check(lib.ni_delta_rule(_ptr(prep), _ptr(chunks), _ptr(state), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(o),

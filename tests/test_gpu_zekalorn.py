@@ -478,16 +478,28 @@ def test_delta_rule_in_runs_of_sixteen_and_token_by_token_agree_with_the_plain_r
     f32 = lambda t: t.to(dev, torch.float32).contiguous()
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
     seq_of_token = i32([s for s, n in enumerate(lens) for _ in range(n)])
-    for what, longest in (("token by token", 1), ("runs of sixteen", max(lens))):
+    for what, in_runs in (("token by token", False), ("runs of sixteen", True)):
         st = f32(state)
         got = K.delta_rule(f32(proj), f32(low), f32(conv), f32(a_log), f32(dt_bias), f32(norm_w), st, seq_of_token, i32(starts),
-                           i32(lens), i32(slots), G, H, dk, dv, taps, 1e-5, torch.float32, max_q_len=longest)
+                           i32(lens), i32(slots), G, H, dk, dv, taps, 1e-5, torch.float32, max_q_len=max(lens), runs=in_runs)
         err = float((got.double().cpu() - want).abs().max() / want.abs().max())
         assert err < 2e-5, (what, "read-out", err)
         err = float((st.double().cpu() - want_state).abs().max() / want_state.abs().max())
         assert err < 2e-5, (what, "state", err)
         untouched = [s for s in range(7) if s not in slots]
         assert torch.equal(st.cpu()[untouched], state.float()[untouched]), what
+    # steps of single tokens (the first kernel moves the convolutions' inputs on): five sequences, three steps
+    lens1, starts1 = [1] * 5, list(range(5))
+    st, st64 = f32(state), state.clone()
+    for step in range(3):
+        rows = slice(5 * step, 5 * step + 5)
+        want, st64 = _plain_delta_step(proj[rows], low[rows], conv, a_log, dt_bias, norm_w, st64, starts1, lens1, slots, G, H, dk, dv, taps, 1e-5)
+        got = K.delta_rule(f32(proj[rows]), f32(low[rows]), f32(conv), f32(a_log), f32(dt_bias), f32(norm_w), st, i32([0, 1, 2, 3, 4]),
+                           i32(starts1), i32(lens1), i32(slots), G, H, dk, dv, taps, 1e-5, torch.float32, max_q_len=1)
+        err = float((got.double().cpu() - want).abs().max() / want.abs().max())
+        assert err < 2e-5, ("single tokens", step, err)
+    err = float((st.double().cpu() - st64).abs().max() / st64.abs().max())
+    assert err < 2e-5, ("single tokens, state", err)
 
 
 # ------------------------------------------------------------------ generation through the entry point
