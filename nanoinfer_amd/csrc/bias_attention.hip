@@ -390,22 +390,32 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     }
 }
 
-// out[row, :] = sum_r acc_r e^(m_r - M) / sum_r l_r e^(m_r - M) over the runs of a row (an empty run has l = 0)
+// out[row, :] = sum_r acc_r e^(m_r - M) / sum_r l_r e^(m_r - M) over the runs of a row (an empty run has l = 0).
+// One wavefront a row; lane r takes run r's maximum and sum (n_runs <= 64), the weights e^(m_r - M) go through LDS,
+// and the sums over the runs then read nothing that depends on an earlier read.
 template <typename T>
-__global__ void merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv) {
+__global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv) {
+    __shared__ float weight[WAVE];
     const size_t row = blockIdx.x;
     const float* p = partial + row * n_runs * (dv + 2);
-    float M = -INFINITY;
-    for (int r = 0; r < n_runs; ++r) M = fmaxf(M, p[r * (dv + 2)]);
-    float L = 0.f;
-    for (int r = 0; r < n_runs; ++r) {
-        const float l = p[r * (dv + 2) + 1];
-        if (l > 0.f) L += l * expf(p[r * (dv + 2)] - M);
+    const int lane = threadIdx.x;
+    float m = -INFINITY, l = 0.f;
+    if (lane < n_runs) {
+        m = p[lane * (dv + 2)];
+        l = p[lane * (dv + 2) + 1];
     }
-    for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+    if (!(l > 0.f)) m = -INFINITY;
+    const float M = wave_max(m);
+    const float w = l > 0.f ? expf(m - M) : 0.f;
+    const float L = wave_sum(l * w);
+    weight[lane] = w;
+    __syncthreads();
+    for (int c = lane; c < dv; c += WAVE) {
         float a = 0.f;
-        for (int r = 0; r < n_runs; ++r)
-            if (p[r * (dv + 2) + 1] > 0.f) a += p[r * (dv + 2) + 2 + c] * expf(p[r * (dv + 2)] - M);
+        for (int r = 0; r < n_runs; ++r) {
+            const float wr = weight[r];
+            if (wr > 0.f) a += p[r * (dv + 2) + 2 + c] * wr;
+        }
         st(out + row * dv + c, a / L);
     }
 }

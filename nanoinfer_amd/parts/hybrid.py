@@ -224,8 +224,10 @@ class BiasAttention(Part):
         chunks = -(-(self.H // self.G) // self.heads_per_chunk)
         # a step of single tokens has tiles of one token: its rows are the heads of a chunk, four a wavefront
         rows = min(self.tile_tokens, ctx.max_q_len) * self.heads_per_chunk
-        waves = min(4, -(-rows // 4))
-        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, ctx.max_context, waves)
+        # all four wavefronts stage the keys and values, also where fewer of them have rows; the keys are cut into
+        # runs by the wavefronts that have rows
+        waves = 4
+        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, ctx.max_context, min(4, -(-rows // 4)))
         ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
         K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H, self.scale,
                          self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves)
