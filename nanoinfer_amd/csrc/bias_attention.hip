@@ -96,6 +96,72 @@ __device__ __forceinline__ void stage_rows(const T* __restrict__ pool, float* __
     }
 }
 
+// The same in two halves, for tiles whose rows are at most four 16-byte pieces a thread: what stage_rows would
+// load, asked for and kept in registers, and its way into LDS afterwards.  Keys and values asked for one after the
+// other and stored after both are on their way together: one round trip to memory a tile instead of two.
+template <typename T> struct StagedRows {
+    RawRow<T, 16 / sizeof(T)> raw[4];
+    bool have[4];
+};
+
+template <typename T>
+__device__ __forceinline__ void stage_ask(const T* __restrict__ pool, StagedRows<T>& x, int size, const int32_t* __restrict__ table,
+                                          int page_size, int G, int g, int k0, int k_last) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int tid = threadIdx.x, threads = blockDim.x;
+    const int per_row = size / VEC, total = KEYS * per_row;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int idx = u * threads + tid;
+        x.have[u] = false;
+        if (idx < total) {
+            const int j = idx / per_row, pc = idx % per_row, key = k0 + j;
+            if (key <= k_last) {
+                const int page = table[key / page_size];
+                if (page >= 0) {
+                    x.raw[u].load(pool + ((static_cast<size_t>(page) * G + g) * page_size + key % page_size) * size + pc * VEC);
+                    x.have[u] = true;
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void stage_put(const StagedRows<T>& x, float* __restrict__ dst, int stride, int size) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int tid = threadIdx.x, threads = blockDim.x;
+    const int per_row = size / VEC, total = KEYS * per_row;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int idx = u * threads + tid;
+        if (idx < total) {
+            float* d = dst + (idx / per_row) * stride + (idx % per_row) * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) d[e] = x.have[u] ? x.raw[u].get(e) : 0.f;
+        }
+    }
+}
+
+// keys and values of a tile into LDS: together where both fit four pieces a thread, else one after the other
+template <typename T>
+__device__ __forceinline__ void stage_tile(const T* __restrict__ kpool, const T* __restrict__ vpool, float* __restrict__ Ks, int dkp,
+                                           int dk, float* __restrict__ Vs, int dvp, int dv, const int32_t* __restrict__ table,
+                                           int page_size, int G, int g, int k0, int k_last, bool k_pieces, bool v_pieces) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int room = 4 * blockDim.x;
+    if (k_pieces && v_pieces && KEYS * (dk / VEC) <= room && KEYS * (dv / VEC) <= room) {
+        StagedRows<T> k, v;
+        stage_ask<T>(kpool, k, dk, table, page_size, G, g, k0, k_last);
+        stage_ask<T>(vpool, v, dv, table, page_size, G, g, k0, k_last);
+        stage_put<T>(k, Ks, dkp, dk);
+        stage_put<T>(v, Vs, dvp, dv);
+        return;
+    }
+    stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, k_last, k_pieces);
+    stage_rows<T>(vpool, Vs, dvp, dv, table, page_size, G, g, k0, k_last, v_pieces);
+}
+
 template <typename T>
 __global__ void __launch_bounds__(WAVES * WAVE)
 bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
@@ -152,8 +218,7 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
     const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
     for (int k0 = k_begin; k0 <= k_last; k0 += KEYS) {
         __syncthreads();                          // the tile before this one has been used by everyone
-        stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, k_last, k_pieces);
-        stage_rows<T>(vpool, Vs, dv, dv, table, page_size, G, g, k0, k_last, v_pieces);
+        stage_tile<T>(kpool, vpool, Ks, dkp, dk, Vs, dv, dv, table, page_size, G, g, k0, k_last, k_pieces, v_pieces);
         __syncthreads();
         // scores of this lane's key for the wavefront's rows
         float s[ROWS_PER_WAVE];
@@ -318,6 +383,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     const float* qrow = Qs + row * dkp + kg * (dk / 4);
     for (int k0 = 0; k0 <= last_pos; k0 += KEYS) {
         __syncthreads();                          // the tile before this one has been used by everyone
+        // one after the other: both in registers at once would cost this kernel its second wavefront a SIMD
         stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, last_pos, k_pieces);
         stage_rows<T>(vpool, Vs, dvp, dv, table, page_size, G, g, k0, last_pos, v_pieces);
         __syncthreads();
