@@ -225,9 +225,44 @@ __global__ void experts_act_kernel(const T* __restrict__ up, const float* __rest
     st(act + i, v);
 }
 
+// the same, eight neighbouring elements a thread (ff a multiple of 8: they are one expert's); the elements of an
+// expert that was not chosen are not read at all
+template <typename T>
+__global__ void experts_act_vec_kernel(const T* __restrict__ up, const float* __restrict__ mix_all, T* __restrict__ act,
+                                       int E, int ff, size_t pieces) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= pieces) return;
+    const size_t i = idx * 8;
+    const size_t width = static_cast<size_t>(E) * ff;
+    const size_t t = i / width;
+    const int e = static_cast<int>((i - t * width) / ff);
+    const float w = mix_all[t * E + e];
+    float v[8];
+    if (w != 0.f) {
+        VecIO<T, 8>::load(up + i, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float u = fmaxf(v[j], 0.f);
+            v[j] = w * (u * u);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = 0.f;
+    }
+    VecIO<T, 8>::store(act + i, v);
+}
+
 NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int dtype, hipStream_t stream) {
     const size_t n = static_cast<size_t>(T) * E * ff;
     if (n == 0) return 0;
+    if (ff % 8 == 0 && aligned16(up, act)) {
+        const size_t pieces = n / 8;
+        if (dtype == 0)
+            experts_act_vec_kernel<float><<<blocks_of(pieces, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, pieces);
+        else
+            experts_act_vec_kernel<bf16_t><<<blocks_of(pieces, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, pieces);
+        return NI_LAUNCH_RESULT();
+    }
     if (dtype == 0)
         experts_act_kernel<float><<<blocks_of(n, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, n);
     else
