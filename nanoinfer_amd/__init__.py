@@ -8,7 +8,9 @@ hand-written HIP kernels under ``csrc/``.
 from . import registry
 from .parts import standard as _standard_parts   # registers the parts
 from .parts import hybrid as _hybrid_parts       # registers the parallel block, the mixers with a memory, routed experts
+from .parts import stateful as _stateful_parts   # registers mixers with a state of fixed size, the windowed attention, the pair-hash embedding
 from .architectures import llama as _llama       # registers LlamaForCausalLM
 from .architectures import zekalorn as _zekalorn  # registers Zekalorn
+from .architectures import fusavik as _fusavik    # registers Fusavik
 
 __version__ = "0.1.0"

@@ -8,6 +8,12 @@
 // row for every distance up to the model's last position), so the kernel needs no logarithm a score.
 // Pools are [page, kv_head, slot_in_page, size] with size dk for keys and dv for values.
 //
+// A window (`window` > 0) narrows what a query sees to its last `window` keys, its own among them, plus the
+// first `keep_first` keys of its sequence, which stay visible for good: j <= i and (i - j < window or j < keep_first).
+// The kernels then walk only the tiles of 64 keys that hold such keys: the tiles of the kept first keys, then the
+// tiles from the one in which the window of the tile's first token starts (`KeyWalk`).  `out_scale` multiplies the
+// normalised output (a mixer that is one of several side by side has a weight of its own).
+//
 // One workgroup of four wavefronts takes a tile of consecutive tokens of one sequence and (a chunk of)
 // the query heads of one kv head: 16 rows of (token, head), four a wavefront.  64 keys and values at a
 // time are staged in LDS as float32 for the whole workgroup; a lane owns one key of the 64 for the
@@ -23,6 +29,27 @@
 #define ROWS (ROWS_PER_WAVE * WAVES)
 #define KEYS 64
 #define MAX_VCHUNKS 4          // value channels a lane owns at most: dv <= 256
+
+// Which tiles of KEYS keys a tile of queries (positions first_pos .. last_pos) walks: step v < kept is tile v (the kept
+// first keys), step v >= kept the tile at `start + (v - kept) * KEYS`.  Without a window: every tile from key 0.
+struct KeyWalk {
+    int kept, start, steps;
+    __device__ __forceinline__ KeyWalk(int first_pos, int last_pos, int window, int keep_first) {
+        kept = 0;
+        start = 0;
+        if (window > 0) {
+            const int lo = max(first_pos - window + 1, 0) / KEYS * KEYS;       // the tile in which the first row's window starts
+            const int kept_end = (min(keep_first, last_pos + 1) + KEYS - 1) / KEYS * KEYS;
+            if (lo > kept_end) { kept = kept_end / KEYS; start = lo; }
+        }
+        steps = kept + (last_pos - start) / KEYS + 1;
+    }
+    __device__ __forceinline__ int first_key(int v) const { return v < kept ? v * KEYS : start + (v - kept) * KEYS; }
+};
+
+__device__ __forceinline__ bool key_seen(int key, int pos, int window, int keep_first) {
+    return key <= pos && (window <= 0 || pos - key < window || key < keep_first);
+}
 
 // keys and values of the step's tokens into their places in the pages
 template <typename T>
@@ -42,6 +69,88 @@ __global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k
         const int g = i / dv, c = i % dv;
         vpool[((static_cast<size_t>(page) * G + g) * page_size + in_page) * dv + c] = row[v_off + i];
     }
+}
+
+// The same for projections that still want their norm and rotation, all of it in float32:
+//   q <- rotate(rmsnorm(q) * wq), k <- rotate(rmsnorm(k) * wk)      the norms run over the WHOLE projection of a token
+//   (all heads at once; a null weight: no norm), the rotation turns channel c < rot/2 of every head together with
+//   channel c + rot/2 by the angle position * freq[c], cos and sin times `amplitude` (a null freq: no rotation);
+//   the channels from `rot` on pass as they are.
+// proj float32 [T, row_stride] holds q [H * dk] | k [G * dk] | v [G * dv]; q goes to q_out [T, H * dk] in the compute
+// type, k and v into their page slots.  One workgroup a token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const int32_t* __restrict__ positions,
+                          const int32_t* __restrict__ slot_mapping, const float* __restrict__ wq, const float* __restrict__ wk,
+                          float eps, const float* __restrict__ freq, int rot, float amplitude, T* __restrict__ q_out,
+                          T* __restrict__ kpool, T* __restrict__ vpool, int H, int G, int dk, int dv, int page_size) {
+    __shared__ float scratch[8];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float* row = proj + static_cast<size_t>(t) * row_stride;
+    const int nq = H * dk, nk = G * dk;
+    float rq = 1.f, rk = 1.f;
+    if (wq) {
+        float ss = 0.f;
+        for (int i = tid; i < nq; i += blockDim.x) ss += row[i] * row[i];
+        rq = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(nq) + eps);
+    }
+    if (wk) {
+        float ss = 0.f;
+        for (int i = tid; i < nk; i += blockDim.x) ss += row[nq + i] * row[nq + i];
+        rk = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(nk) + eps);
+    }
+    const float pos = static_cast<float>(positions[t]);
+    const int half = rot / 2;
+    const int slot = slot_mapping ? slot_mapping[t] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0, in_page = slot >= 0 ? slot % page_size : 0;
+    for (int i = tid; i < nq + nk; i += blockDim.x) {
+        const bool is_q = i < nq;
+        const int j = is_q ? i : i - nq;                 // index inside the projection
+        const float* src = is_q ? row : row + nq;
+        const float* w = is_q ? wq : wk;
+        const float r = is_q ? rq : rk;
+        const int c = j % dk;
+        float v = src[j] * r * (w ? w[j] : 1.f);
+        if (freq && c < rot) {
+            const int jp = c < half ? j + half : j - half;
+            const float other = src[jp] * r * (w ? w[jp] : 1.f);
+            float sn, cs;
+            sincosf(pos * freq[c < half ? c : c - half], &sn, &cs);
+            sn *= amplitude;
+            cs *= amplitude;
+            v = c < half ? v * cs - other * sn : v * cs + other * sn;
+        }
+        if (is_q) {
+            st(q_out + static_cast<size_t>(t) * nq + j, v);
+        } else if (slot >= 0) {
+            const int g = j / dk;
+            st(kpool + ((static_cast<size_t>(page) * G + g) * page_size + in_page) * dk + c, v);
+        }
+    }
+    if (slot >= 0) {
+        const float* vsrc = row + nq + nk;
+        for (int i = tid; i < G * dv; i += blockDim.x) {
+            const int g = i / dv, c = i % dv;
+            st(vpool + ((static_cast<size_t>(page) * G + g) * page_size + in_page) * dv + c, vsrc[i]);
+        }
+    }
+}
+
+NI_EXPORT int ni_qk_norm_rope_store(const void* proj, int row_stride, const void* positions, const void* slot_mapping,
+                                    const void* wq, const void* wk, float eps, const void* freq, int rot, float amplitude,
+                                    void* q_out, void* kpool, void* vpool, int T, int H, int G, int dk, int dv, int page_size,
+                                    int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (rot < 0 || rot > dk || rot % 2 || row_stride < H * dk + G * dk + G * dv) return -1;
+    if (dtype == 0)
+        qk_norm_rope_store_kernel<float><<<T, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
+            (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
+            (float*)q_out, (float*)kpool, (float*)vpool, H, G, dk, dv, page_size);
+    else
+        qk_norm_rope_store_kernel<bf16_t><<<T, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
+            (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
+            (bf16_t*)q_out, (bf16_t*)kpool, (bf16_t*)vpool, H, G, dk, dv, page_size);
+    return NI_LAUNCH_RESULT();
 }
 
 // 64 rows of a pool (keys or values of one kv head) from their pages into LDS as float32, row stride `stride`.
@@ -168,7 +277,8 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
                       const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
                       int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk, int n_runs,
-                      float* __restrict__ partial, bool k_pieces, bool v_pieces, int dkp) {
+                      float* __restrict__ partial, bool k_pieces, bool v_pieces, int dkp, int window, int keep_first,
+                      float out_scale) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     // a lane reads its key's row: the stride is the row plus four floats where rows are whole 16-byte pieces (read
     // as such), plus one otherwise; both spread the lanes over the banks
@@ -213,10 +323,13 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
         for (int cc = 0; cc < MAX_VCHUNKS; ++cc) acc[rr][cc] = 0.f;
     }
     const int last_pos = first_pos + n_tok - 1;
-    const int span = ((last_pos + n_runs) / n_runs + KEYS - 1) / KEYS * KEYS;      // keys of a run: whole tiles of 64
-    const int k_begin = run * span, k_last = std::min(last_pos, k_begin + span - 1);
+    const KeyWalk walk(first_pos, last_pos, window, keep_first);
+    const int per_run = (walk.steps + n_runs - 1) / n_runs;                        // tiles of 64 keys a run
+    const int v_end = std::min(walk.steps, (run + 1) * per_run);
+    const int k_last = last_pos;
     const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
-    for (int k0 = k_begin; k0 <= k_last; k0 += KEYS) {
+    for (int v = run * per_run; v < v_end; ++v) {
+        const int k0 = walk.first_key(v);
         __syncthreads();                          // the tile before this one has been used by everyone
         stage_tile<T>(kpool, vpool, Ks, dkp, dk, Vs, dv, dv, table, page_size, G, g, k0, k_last, k_pieces, v_pieces);
         __syncthreads();
@@ -250,14 +363,15 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
             alpha[rr] = 1.f;
             if (!valid[rr]) { prow[rr * KEYS + lane] = 0.f; continue; }          // the same for the whole wavefront
             if (k0 > pos[rr]) { prow[rr * KEYS + lane] = 0.f; continue; }        // the same for the whole wavefront
-            const bool seen = key <= pos[rr] && key <= k_last;
+            const bool seen = key_seen(key, pos[rr], window, keep_first);
             float sc = -INFINITY;
             if (seen) {
                 const int back = std::min(pos[rr] - key, distances - 1);
                 sc = s[rr] * factor[rr] + (bias ? bias[static_cast<size_t>(back) * H + head[rr]] : 0.f);
             }
-            const float m_new = fmaxf(m[rr], wave_max(sc));      // finite: key k0 <= pos is seen
-            alpha[rr] = expf(m[rr] - m_new);                      // 0 at the first tile
+            const float m_new = fmaxf(m[rr], wave_max(sc));
+            if (m_new == -INFINITY) { prow[rr * KEYS + lane] = 0.f; continue; }   // no key of this row so far (a window that starts later)
+            alpha[rr] = expf(m[rr] - m_new);                      // 0 at the row's first keys
             const float p = seen ? expf(sc - m_new) : 0.f;
             l[rr] = l[rr] * alpha[rr] + wave_sum(p);
             m[rr] = m_new;
@@ -300,7 +414,7 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
             continue;
         }
         T* orow = out + static_cast<size_t>(first_row + r / heads_here) * (H * dv) + head[rr] * dv;
-        const float inv = 1.0f / l[rr];
+        const float inv = out_scale / l[rr];
 #pragma unroll
         for (int cc = 0; cc < MAX_VCHUNKS; ++cc) {
             const int c = lane + cc * WAVE;
@@ -341,7 +455,8 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
                            const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
                            const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances,
                            T* __restrict__ out, int H, int G, int dk, int dv, int page_size, float scale, float temp_coef,
-                           int temp_every, int heads_per_chunk, bool k_pieces, bool v_pieces) {
+                           int temp_every, int heads_per_chunk, bool k_pieces, bool v_pieces, int window, int keep_first,
+                           float out_scale) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dkp = dk + 4, dvp = dv + 4;         // strides that spread the sixteen rows of a read over the banks
     float* Qs = lds;                              // [MROWS][dkp]
@@ -381,7 +496,9 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     const int last_pos = first_pos + n_tok - 1;
     const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
     const float* qrow = Qs + row * dkp + kg * (dk / 4);
-    for (int k0 = 0; k0 <= last_pos; k0 += KEYS) {
+    const KeyWalk walk(first_pos, last_pos, window, keep_first);
+    for (int v = 0; v < walk.steps; ++v) {
+        const int k0 = walk.first_key(v);
         __syncthreads();                          // the tile before this one has been used by everyone
         // one after the other: both in registers at once would cost this kernel its second wavefront a SIMD
         stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, last_pos, k_pieces);
@@ -409,7 +526,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
             for (int r = 0; r < 4; ++r) {
                 const int key = k0 + 16 * j + 4 * kg + r;
                 float v = -INFINITY;
-                if (valid && key <= pos) {
+                if (valid && key_seen(key, pos, window, keep_first)) {
                     const int back = std::min(pos - key, distances - 1);
                     v = sc[j][r] * factor + (bias ? bias[static_cast<size_t>(back) * H + head] : 0.f);
                 }
@@ -446,7 +563,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     }
     if (!valid) return;
     T* orow = out + static_cast<size_t>(first_row + row / heads_here) * (H * dv) + head * dv + 4 * kg;
-    const float inv = 1.0f / l;
+    const float inv = out_scale / l;
 #pragma unroll
     for (int db = 0; db < MAX_VCHUNKS * 4; ++db) {
         if (db < dvb) {
@@ -460,7 +577,8 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
 // One wavefront a row; lane r takes run r's maximum and sum (n_runs <= 64), the weights e^(m_r - M) go through LDS,
 // and the sums over the runs then read nothing that depends on an earlier read.
 template <typename T>
-__global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv) {
+__global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv,
+                                                          float out_scale) {
     __shared__ float weight[WAVE];
     const size_t row = blockIdx.x;
     const float* p = partial + row * n_runs * (dv + 2);
@@ -482,7 +600,7 @@ __global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restric
             const float wr = weight[r];
             if (wr > 0.f) a += p[r * (dv + 2) + 2 + c] * wr;
         }
-        st(out + row * dv + c, a / L);
+        st(out + row * dv + c, a * out_scale / L);
     }
 }
 
@@ -503,8 +621,10 @@ NI_EXPORT int ni_bias_attention_rows() { return ROWS; }
 NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
                                 int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias, int distances, void* out,
                                 int H, int G, int dk, int dv, int page_size, float scale, float temp_coef, int temp_every,
-                                int heads_per_chunk, int n_runs, void* partial, int n_rows, int waves, int dtype, hipStream_t stream) {
+                                int heads_per_chunk, int n_runs, void* partial, int n_rows, int waves, int window, int keep_first,
+                                float out_scale, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
+    if (window < 0 || keep_first < 0) return -1;
     if (dv > MAX_VCHUNKS * WAVE || H % G || heads_per_chunk < 1 || heads_per_chunk > ROWS) return -1;
     const int group = H / G;
     const int dkp = dk % 4 == 0 ? dk + 4 : dk + 1;
@@ -526,8 +646,8 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<float><<<grid, waves * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp);
-        if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale);
+        if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv, out_scale);
     } else {
         static size_t allowed = 48 * 1024;
         if (lds > allowed && (allowed = lds))
@@ -536,8 +656,8 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<bf16_t><<<grid, waves * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp);
-        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale);
+        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv, out_scale);
     }
     return NI_LAUNCH_RESULT();
 }
@@ -553,8 +673,10 @@ NI_EXPORT int ni_bias_attention_mfma_rows(int dk, int dv) {
 NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void* kpool, const void* vpool, const void* block_table,
                                      int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias,
                                      int distances, void* out, int H, int G, int dk, int dv, int page_size, float scale,
-                                     float temp_coef, int temp_every, int heads_per_chunk, int dtype, hipStream_t stream) {
+                                     float temp_coef, int temp_every, int heads_per_chunk, int window, int keep_first,
+                                     float out_scale, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
+    if (window < 0 || keep_first < 0) return -1;
     if (!ni_bias_attention_mfma_rows(dk, dv) || H % G || heads_per_chunk < 1 || heads_per_chunk > MROWS) return -1;
     const int group = H / G;
     const size_t lds = (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + static_cast<size_t>(KEYS) * (dv + 4)) * sizeof(float);
@@ -571,7 +693,7 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
         bias_attention_mfma_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size,
-            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces);
+            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale);
     } else {
         static size_t allowed = 48 * 1024;
         if (lds > allowed && (allowed = lds))
@@ -580,7 +702,7 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
         bias_attention_mfma_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size,
-            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces);
+            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale);
     }
     return NI_LAUNCH_RESULT();
 }

@@ -125,6 +125,7 @@ SAMPLING = ("ni_sampling", ["sampling.hip"], {})
 SKINNY = ("ni_skinny_gemm", ["gemv.hip"], {})
 STREAM_OPS = ("ni_stream_ops", ["stream_ops.hip"], {})
 BIAS_ATTENTION = ("ni_bias_attention", ["bias_attention.hip"], {})
+STATE_MIXERS = ("ni_state_mixers", ["state_mixers.hip"], {})
 COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 256)
 COMMON_DELTA_KEY_SIZES = (16, 20, 32, 48, 64, 96, 128)
 
@@ -169,7 +170,7 @@ def attention_mfma_f32_target(head_dim: int):
 def build_all(head_dims: Iterable[int] = COMMON_HEAD_DIMS, force: bool = True, verbose: bool = True,
               jobs: Optional[int] = None, delta_key_sizes: Iterable[int] = COMMON_DELTA_KEY_SIZES) -> List[str]:
     """Compile every library (attention for the given head sizes, the delta rule for the given key sizes)."""
-    targets = [CORE, SAMPLING, SKINNY, STREAM_OPS, BIAS_ATTENTION] + [delta_rule_target(k) for k in delta_key_sizes] + \
+    targets = [CORE, SAMPLING, SKINNY, STREAM_OPS, BIAS_ATTENTION, STATE_MIXERS] + [delta_rule_target(k) for k in delta_key_sizes] + \
         [attention_target(h) for h in head_dims] + \
         [attention_mfma_target(h) for h in head_dims] + \
         [attention_mfma_f32_target(h) for h in head_dims]

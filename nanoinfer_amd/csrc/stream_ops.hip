@@ -54,6 +54,74 @@ NI_EXPORT int ni_embed_scaled(const void* ids, const void* positions, const void
     return NI_LAUNCH_RESULT();
 }
 
+// ---------------------------------------------------------------- embedding: row * scale + row of a table of token pairs
+// out[t] = table[ids[t]] * scale + pairs[(prev * mul_prev + ids[t] * mul_cur) mod buckets], prev the token before
+// ids[t] in its sequence; a sequence's first token (position 0) takes row `buckets`.  The token before the first
+// row of a portion is what `last_token[slot]` holds: remember_last_kernel leaves every sequence's last token there
+// after the rows have been read (a launch of its own: the first row of a portion must not see it).
+template <typename T>
+__global__ void embed_pair_hash_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ positions,
+                                       const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
+                                       const int32_t* __restrict__ state_slot, const int32_t* __restrict__ last_token,
+                                       const T* __restrict__ table, const T* __restrict__ pairs, float* __restrict__ out,
+                                       int d, int vocab, int buckets, long long mul_prev, long long mul_cur, float scale) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    if (id < 0 || id >= vocab) return;      // unreachable after the host's check
+    int row = buckets;
+    if (positions[t] > 0) {
+        const int s = seq_of_token[t];
+        const int prev = (t == q_start[s]) ? last_token[state_slot[s]] : ids[t - 1];
+        long long r = (static_cast<long long>(prev) * mul_prev + static_cast<long long>(id) * mul_cur) % buckets;
+        if (r < 0) r += buckets;
+        row = static_cast<int>(r);
+    }
+    const T* erow = table + static_cast<size_t>(id) * d;
+    const T* prow = pairs + static_cast<size_t>(row) * d;
+    float* o = out + static_cast<size_t>(t) * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = ld(erow + i) * scale + ld(prow + i);
+}
+
+__global__ void remember_last_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ q_start,
+                                     const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot,
+                                     int32_t* __restrict__ last_token, int B) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < B && q_len[b] > 0) last_token[state_slot[b]] = ids[q_start[b] + q_len[b] - 1];
+}
+
+NI_EXPORT int ni_embed_pair_hash(const void* ids, const void* positions, const void* seq_of_token, const void* q_start,
+                                 const void* q_len, const void* state_slot, void* last_token, const void* table,
+                                 const void* pairs, void* out, int T, int B, int d, int vocab, int buckets, long long mul_prev,
+                                 long long mul_cur, float scale, int dtype, hipStream_t stream) {
+    if (T <= 0 || B <= 0) return 0;
+    if (buckets < 1) return -1;
+    if (dtype == 0)
+        embed_pair_hash_kernel<float><<<T, 256, 0, stream>>>((const int32_t*)ids, (const int32_t*)positions, (const int32_t*)seq_of_token,
+            (const int32_t*)q_start, (const int32_t*)state_slot, (const int32_t*)last_token, (const float*)table, (const float*)pairs,
+            (float*)out, d, vocab, buckets, mul_prev, mul_cur, scale);
+    else
+        embed_pair_hash_kernel<bf16_t><<<T, 256, 0, stream>>>((const int32_t*)ids, (const int32_t*)positions, (const int32_t*)seq_of_token,
+            (const int32_t*)q_start, (const int32_t*)state_slot, (const int32_t*)last_token, (const bf16_t*)table, (const bf16_t*)pairs,
+            (float*)out, d, vocab, buckets, mul_prev, mul_cur, scale);
+    remember_last_kernel<<<blocks_of(B, 64), 64, 0, stream>>>((const int32_t*)ids, (const int32_t*)q_start, (const int32_t*)q_len,
+                                                               (const int32_t*)state_slot, (int32_t*)last_token, B);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- h[t, :] += extra[t, :] + vec   (extra may be absent)
+__global__ void add_rows_vector_kernel(float* __restrict__ h, const float* __restrict__ extra, const float* __restrict__ vec,
+                                       int d, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) h[i] = (extra ? h[i] + extra[i] : h[i]) + vec[i % d];
+}
+
+NI_EXPORT int ni_add_rows_vector(void* h, const void* extra, const void* vec, int T, int d, hipStream_t stream) {
+    const size_t n = static_cast<size_t>(T) * d;
+    if (n == 0) return 0;
+    add_rows_vector_kernel<<<blocks_of(n, 256), 256, 0, stream>>>((float*)h, (const float*)extra, (const float*)vec, d, n);
+    return NI_LAUNCH_RESULT();
+}
+
 // ---------------------------------------------------------------- h[t, :] += vec
 __global__ void add_vector_kernel(float* __restrict__ h, const float* __restrict__ vec, int d, size_t n) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -153,13 +221,16 @@ NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int
 }
 
 // ---------------------------------------------------------------- the router's choice
-// z float32 [T, E]: the `top` largest logits of a row (the lower index on equal logits), their softmax
-// among themselves.  chosen int32 [T, top], mix float32 [T, top], and (if asked for) the same as a row
-// over all experts, zero where an expert was not chosen.
+// z float32 [T, E]: the `top` largest logits of a row (the lower index on equal logits) and their weights:
+// the softmax among the chosen (`over_all` 0) or the softmax over all E experts, not renormalised (`over_all` 1).
+// With `n_groups` > 1 the experts form that many equal groups of neighbours; a group counts as much as its
+// largest logit, and only experts of the `keep` best groups (the lower index on equal ones) can be chosen.
+// chosen int32 [T, top], mix float32 [T, top], and (if asked for) the same as a row over all experts, zero where
+// an expert was not chosen.
 // One wavefront a row: a lane keeps the logits of experts lane, lane + 64, ...; each of the `top` rounds finds the
 // largest logit not yet taken (the lowest index among equal ones) by two butterflies over the lanes.
 __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen, float* __restrict__ mix,
-                                 float* __restrict__ mix_all, int T, int E, int top) {
+                                 float* __restrict__ mix_all, int T, int E, int top, int over_all, int n_groups, int keep) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* row = z + static_cast<size_t>(t) * E;
     int32_t* c = chosen + static_cast<size_t>(t) * top;
@@ -170,22 +241,56 @@ __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restric
         for (int e = lane; e < E; e += WAVE) mix_all[static_cast<size_t>(t) * E + e] = 0.f;
         __threadfence_block();
     }
+    unsigned long long open_groups = ~0ull;       // bit g: experts of group g may be chosen
+    const int per_group = E / max(n_groups, 1);
+    if (n_groups > 1) {
+        // lane g ends up with the largest logit of group g
+        float mine = -INFINITY;
+        for (int g = 0; g < n_groups; ++g) {
+            float v = -INFINITY;
+            for (int e = lane; e < E; e += WAVE)
+                if (e / per_group == g) { const float ze = row[e]; if (ze == ze) v = fmaxf(v, ze); }
+            v = wave_max(v);
+            if (lane == g) mine = v;
+        }
+        open_groups = 0ull;
+        bool used = lane >= n_groups;
+        for (int k = 0; k < keep; ++k) {
+            const float v = used ? -INFINITY : mine;
+            const float vmax = wave_max(v);
+            int cand = (!used && v == vmax) ? lane : 0x7fffffff;
+#pragma unroll
+            for (int off = WAVE / 2; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, WAVE));
+            if (cand == 0x7fffffff) break;        // unreachable: keep <= n_groups
+            if (cand == lane) used = true;
+            open_groups |= 1ull << cand;
+        }
+    }
+    if (over_all) {                 // the softmax runs over every expert, chosen or not
+        float v = -INFINITY;
+        for (int e = lane; e < E; e += WAVE) { const float ze = row[e]; if (ze == ze) v = fmaxf(v, ze); }
+        best = wave_max(v);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += WAVE) { const float ze = row[e]; if (ze == ze) sum += expf(ze - best); }
+        total = wave_sum(sum);
+    }
     for (int k = 0; k < top; ++k) {
         float v = -INFINITY;
         int at = 0x7fffffff;
         for (int e = lane; e < E; e += WAVE) {
             const bool taken = (taken_mask >> (e / WAVE)) & 1u;
+            const bool open = (open_groups >> (n_groups > 1 ? e / per_group : 0)) & 1ull;
             float ze = row[e];
             if (!(ze == ze)) ze = -INFINITY;       // a logit that is no number is never preferred
-            if (!taken && (at == 0x7fffffff || ze > v)) { at = e; v = ze; }
+            if (!taken && open && (at == 0x7fffffff || ze > v)) { at = e; v = ze; }
         }
         const float vmax = wave_max(v);
         int cand = (at != 0x7fffffff && v == vmax) ? at : 0x7fffffff;
 #pragma unroll
         for (int off = WAVE / 2; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, WAVE));
-        if (k == 0) best = vmax;
+        if (k == 0 && !over_all) best = vmax;
         const float w = expf(vmax - best);
-        total += w;
+        if (!over_all) total += w;
         if (cand % WAVE == lane) taken_mask |= 1u << (cand / WAVE);
         if (lane == 0) { c[k] = cand; m[k] = w; }
     }
@@ -198,10 +303,13 @@ __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restric
     }
 }
 
-NI_EXPORT int ni_route_top(const void* z, void* chosen, void* mix, void* mix_all, int T, int E, int top, hipStream_t stream) {
+NI_EXPORT int ni_route_top(const void* z, void* chosen, void* mix, void* mix_all, int T, int E, int top, int over_all,
+                           int n_groups, int keep, hipStream_t stream) {
     if (T <= 0) return 0;
     if (top < 1 || top > E || E > 32 * WAVE) return -1;
-    route_top_kernel<<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top);
+    if (n_groups < 1 || n_groups > WAVE || E % n_groups || keep < 1 || keep > n_groups || top > E / n_groups * keep) return -1;
+    route_top_kernel<<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
+                                             over_all, n_groups, keep);
     return NI_LAUNCH_RESULT();
 }
 
@@ -252,9 +360,35 @@ __global__ void experts_act_vec_kernel(const T* __restrict__ up, const float* __
     VecIO<T, 8>::store(act + i, v);
 }
 
-NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int dtype, hipStream_t stream) {
+// the gated form: an expert's rows of `up` are [gate: ff | up: ff], act[t, e * ff + i] = mix_all[t, e] * silu(gate) * up
+template <typename T>
+__global__ void experts_act_gated_kernel(const T* __restrict__ up, const float* __restrict__ mix_all, T* __restrict__ act,
+                                         int E, int ff, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t width = static_cast<size_t>(E) * ff;
+    const size_t t = i / width;
+    const int e = static_cast<int>((i % width) / ff), c = static_cast<int>(i % ff);
+    const float w = mix_all[t * E + e];
+    float v = 0.f;
+    if (w != 0.f) {
+        const T* src = up + (t * E + e) * 2 * static_cast<size_t>(ff);
+        const float g = ld(src + c), u = ld(src + ff + c);
+        v = w * (g / (1.0f + expf(-g))) * u;
+    }
+    st(act + i, v);
+}
+
+NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int gated, int dtype, hipStream_t stream) {
     const size_t n = static_cast<size_t>(T) * E * ff;
     if (n == 0) return 0;
+    if (gated) {
+        if (dtype == 0)
+            experts_act_gated_kernel<float><<<blocks_of(n, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, n);
+        else
+            experts_act_gated_kernel<bf16_t><<<blocks_of(n, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, n);
+        return NI_LAUNCH_RESULT();
+    }
     if (ff % 8 == 0 && aligned16(up, act)) {
         const size_t pieces = n / 8;
         if (dtype == 0)
@@ -277,9 +411,10 @@ NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int
 //   out[t, r] = sum_k mix[t, k] * W_down[r, chosen[t, k] * ff : +ff] . hid[t * top + k, :]
 // A wavefront takes R neighbouring rows at once, with a sum of its own for each: the loads of the R rows are in
 // flight together, and the input row is read once for all of them.
-template <typename T, int R>
+template <typename T, int R, bool GATED>
 __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restrict__ w_up, const int32_t* __restrict__ chosen,
                                       float* __restrict__ hid, int d, int ff, int top, bool vec) {
+    // GATED: an expert owns 2 ff rows of w_up, its gate rows and then its up rows; hid = silu(gate . x) * (up . x)
     const int pair = blockIdx.x;                 // t * top + k
     const int t = pair / top;
     const int e = chosen[pair];
@@ -287,20 +422,25 @@ __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restri
     const T* xr = x + static_cast<size_t>(t) * d;
     const int i0 = (blockIdx.y * waves + wave) * R;
     if (i0 >= ff) return;
-    const T* wr[R];
+    constexpr int RR = GATED ? 2 * R : R;        // rows of the matrix a wavefront walks: R, or R gate rows and R up rows
+    const T* wr[RR];
 #pragma unroll
-    for (int u = 0; u < R; ++u) wr[u] = w_up + (static_cast<size_t>(e) * ff + min(i0 + u, ff - 1)) * d;
-    float s[R];
+    for (int u = 0; u < R; ++u) {
+        const size_t first = static_cast<size_t>(e) * (GATED ? 2 * ff : ff) + min(i0 + u, ff - 1);
+        wr[u] = w_up + first * d;
+        if constexpr (GATED) wr[R + u] = w_up + (first + ff) * d;
+    }
+    float s[RR];
 #pragma unroll
-    for (int u = 0; u < R; ++u) s[u] = 0.f;
+    for (int u = 0; u < RR; ++u) s[u] = 0.f;
     if (vec) {          // eight elements a lane and load: a wavefront takes 512 neighbouring elements of a row at once
         for (int c = lane * 8; c < d; c += WAVE * 8) {
-            float wv[R][8], xv[8];
+            float wv[RR][8], xv[8];
 #pragma unroll
-            for (int u = 0; u < R; ++u) VecIO<T, 8>::load(wr[u] + c, wv[u]);
+            for (int u = 0; u < RR; ++u) VecIO<T, 8>::load(wr[u] + c, wv[u]);
             VecIO<T, 8>::load(xr + c, xv);
 #pragma unroll
-            for (int u = 0; u < R; ++u)
+            for (int u = 0; u < RR; ++u)
 #pragma unroll
                 for (int j = 0; j < 8; ++j) s[u] += wv[u][j] * xv[j];
         }
@@ -308,15 +448,22 @@ __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restri
         for (int c = lane; c < d; c += WAVE) {
             const float xv = ld(xr + c);
 #pragma unroll
-            for (int u = 0; u < R; ++u) s[u] += ld(wr[u] + c) * xv;
+            for (int u = 0; u < RR; ++u) s[u] += ld(wr[u] + c) * xv;
         }
     }
 #pragma unroll
+    for (int u = 0; u < RR; ++u) s[u] = wave_sum(s[u]);
+#pragma unroll
     for (int u = 0; u < R; ++u) {
-        const float v = wave_sum(s[u]);
         if (lane == 0 && i0 + u < ff) {
-            const float a = fmaxf(v, 0.f);
-            hid[static_cast<size_t>(pair) * ff + i0 + u] = a * a;
+            float a;
+            if constexpr (GATED) {
+                a = s[u] / (1.0f + expf(-s[u])) * s[R + u];
+            } else {
+                a = fmaxf(s[u], 0.f);
+                a = a * a;
+            }
+            hid[static_cast<size_t>(pair) * ff + i0 + u] = a;
         }
     }
 }
@@ -373,29 +520,36 @@ __global__ void experts_down_few_kernel(const float* __restrict__ hid, const T* 
 
 template <typename T, int R>
 static void launch_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
-                               void* hid, void* out, int T_, int d, int ff, int E, int top, bool vec_up, bool vec_down,
+                               void* hid, void* out, int T_, int d, int ff, int E, int top, bool gated, bool vec_up, bool vec_down,
                                hipStream_t stream) {
     constexpr int rows = 4 * R;                  // four wavefronts a workgroup
     dim3 g1(T_ * top, (ff + rows - 1) / rows), g2(T_, (d + rows - 1) / rows);
-    experts_up_few_kernel<T, R><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up);
+    if (gated)
+        experts_up_few_kernel<T, R, true><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up);
+    else
+        experts_up_few_kernel<T, R, false><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up);
     experts_down_few_kernel<T, R><<<g2, 256, 0, stream>>>((const float*)hid, (const T*)w_down, (const int32_t*)chosen,
                                                           (const float*)mix, (float*)out, d, ff, E, top, vec_down);
 }
 
+// `gated` 0: w_up [E * ff, d], hid = relu(.)^2; 1: w_up [E * 2 ff, d] (an expert's gate rows, then its up rows),
+// hid = silu(gate) * up
 NI_EXPORT int ni_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
-                             void* hid, void* out, int T, int d, int ff, int E, int top, int dtype, hipStream_t stream) {
+                             void* hid, void* out, int T, int d, int ff, int E, int top, int gated, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
     // rows of whole 16-byte (bfloat16) or 32-byte (float32) pieces that start on such a piece are read in pieces
     const bool vec_up = d % 8 == 0 && aligned16(x, w_up);
     const bool vec_down = ff % 8 == 0 && aligned16(w_down, hid);
     // four rows a wavefront where that still leaves the second kernel a workgroup for every compute unit, else two
-    const bool four = static_cast<long long>(T) * ((d + 15) / 16) >= 256;
+    // (the gated form walks twice the rows in its first kernel and keeps to two)
+    const bool four = !gated && static_cast<long long>(T) * ((d + 15) / 16) >= 256;
+    const bool g = gated != 0;
     if (dtype == 0) {
-        if (four) launch_experts_few<float, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
-        else launch_experts_few<float, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
+        if (four) launch_experts_few<float, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, g, vec_up, vec_down, stream);
+        else launch_experts_few<float, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, g, vec_up, vec_down, stream);
     } else {
-        if (four) launch_experts_few<bf16_t, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
-        else launch_experts_few<bf16_t, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, vec_up, vec_down, stream);
+        if (four) launch_experts_few<bf16_t, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, g, vec_up, vec_down, stream);
+        else launch_experts_few<bf16_t, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, g, vec_up, vec_down, stream);
     }
     return NI_LAUNCH_RESULT();
 }

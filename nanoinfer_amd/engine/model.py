@@ -35,6 +35,13 @@ class Model:
             if run.enter is not None and self.pass_input is None:
                 raise ValueError(f"an entry of the order adds row {run.enter} of a pass input, the model has none")
         self._needs: Dict[int, CacheNeed] = {}
+        # an embedding that keeps something per request (the token before a portion's first) gets a cache of its
+        # own behind the layers' and is handed it with every step
+        self._embedding_cache = None
+        need = getattr(self.embedding, "cache_need", None)
+        if need is not None and need() is not None:
+            self._embedding_cache = spec.num_caches()
+            self._needs[self._embedding_cache] = need()
         writers = set()
         for run in spec.order:
             need = self.blocks[run.block].cache_need()
@@ -76,7 +83,12 @@ class Model:
         (None when no row is wanted; the caches are filled all the same).  ``logits_out``: float32
         [at least as many rows, vocab] whose first rows are to take the logits, for a head that
         ``writes_into`` a given tensor (any other head returns a tensor of its own)."""
-        h = self.embedding.forward(ctx.token_ids, ctx)
+        if self._embedding_cache is not None:
+            h = self.embedding.forward(ctx.token_ids, ctx, cache=layer_cache(self._embedding_cache, True))
+        else:
+            h = self.embedding.forward(ctx.token_ids, ctx)
+        # a pass input that adds the embedding's output again is given a copy of it (the stream itself moves on)
+        embedded = h.clone() if getattr(self.pass_input, "wants_embedding", False) else None
         pending = None
         order = self.spec.order
         T = h.shape[0]
@@ -87,7 +99,7 @@ class Model:
                 if pending is not None:        # the stream has to be complete before a row is added to it
                     h = self.pass_input.settle(h, pending_for(None, pending, self.rt.dtype))
                     pending = None
-                h = self.pass_input.forward(h, run.enter)
+                h = self.pass_input.forward(h, run.enter) if embedded is None else self.pass_input.forward(h, run.enter, embedded)
             # what the block behind this one would like to find beside the stream (its first norm's input half
             # done by this block's last product), if both blocks know of that
             wants = getattr(self.blocks[order[i + 1].block], "wants_scaled", None) if i + 1 < len(order) else None

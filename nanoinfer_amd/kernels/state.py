@@ -1,0 +1,154 @@
+"""Python face of the kernels in ``csrc/state_mixers.hip``: linear attention with one decay a head, and the
+selective scan with its short convolution.  Their memory of the past is a float32 row of the cache manager's
+state slots.  Shapes, types and devices are checked here, on the host, before a kernel is launched.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from ..csrc import build as _build
+from . import _check, _gpu, _load, _need, _ptr, _stream, dtype_code
+
+_size_t = ctypes.c_size_t
+_float = ctypes.c_float
+
+
+def state_mixers_lib() -> ctypes.CDLL:
+    return _load(_build.STATE_MIXERS)
+
+
+def _per_seq(q_start, q_len, state_slot) -> int:
+    B = q_start.shape[0]
+    for name, t in (("q_start", q_start), ("q_len", q_len), ("state_slot", state_slot)):
+        _need(t.is_cuda and t.dtype == torch.int32 and tuple(t.shape) == (B,), f"{name} must be int32 [{B}] on the GPU")
+    return B
+
+
+def _state(state: torch.Tensor) -> int:
+    _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous(),
+          "state must be float32 [slots, n] on the GPU")
+    return state.shape[1]
+
+
+def _pow2_parts(n: int, per: int) -> int:
+    parts = 1
+    while parts * per < n:
+        parts *= 2
+    return parts
+
+
+def decay_state_floats(heads: int, dk: int, dv: int) -> int:
+    """Floats of one request's state of :func:`decay_attention`: [heads][dv][dk rounded up to 8 * a power of two]."""
+    parts = _pow2_parts(dk, 8)
+    _need(parts <= 64, f"keys of {dk} channels are more than the kernel's 512")
+    return heads * dv * parts * 8
+
+
+def scan_state_floats(inner: int, n: int) -> int:
+    """Floats of one request's recurrent state of :func:`selective_scan`: [inner][n rounded up to 4 * a power of two]."""
+    parts = _pow2_parts(n, 4)
+    _need(parts <= 64, f"{n} numbers a channel are more than the kernel's 256")
+    return inner * parts * 4
+
+
+def silu_rows(x: torch.Tensor, n: int) -> torch.Tensor:
+    """``silu`` of the first ``n`` columns of every row of ``x`` float32 [T, >= n], as float32 [T, n]."""
+    T, width = x.shape
+    _gpu(x, "x", torch.float32)
+    _need(0 < n <= width, "more columns than the rows have")
+    out = torch.empty(T, n, dtype=torch.float32, device=x.device)
+    _check(state_mixers_lib().ni_silu_rows(_ptr(x), width, _ptr(out), T, n, _stream()), "silu_rows")
+    return out
+
+
+def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                    state_slot: torch.Tensor, H: int, dk: int, dv: int) -> torch.Tensor:
+    """Per head ``S <- decay[h] S + k v^T; o = S^T q`` over the rows of every sequence of the step, in order.
+    ``act`` float32 [T, 2 H dk + H dv]: q | k | v after their activation; ``state`` float32 [slots, >=
+    decay_state_floats(H, dk, dv)], moved on by this call.  Returns ``o`` float32 [T, H dv]."""
+    T, width = act.shape
+    _gpu(act, "act", torch.float32)
+    _need(width == 2 * H * dk + H * dv, "act is not q | k | v of these sizes")
+    _gpu(decay, "decay", torch.float32, (H,))
+    stride = _state(state)
+    _need(stride >= decay_state_floats(H, dk, dv), "the state is too small")
+    B = _per_seq(q_start, q_len, state_slot)
+    out = torch.empty(T, H * dv, dtype=torch.float32, device=act.device)
+    _check(state_mixers_lib().ni_decay_attention(_ptr(act), width, _ptr(decay), _ptr(state), _size_t(stride), _ptr(q_start),
+                                                 _ptr(q_len), _ptr(state_slot), _ptr(out), T, B, H, dk, dv, _stream()),
+           "decay_attention")
+    return out
+
+
+def gated_rmsnorm(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, weight: torch.Tensor, eps: float, out_scale: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """``o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate) * out_scale`` row by row; the gate's pre-activations are
+    the columns ``gate_col ..`` of ``gate_rows`` float32 [T, wide]."""
+    T, n = o.shape
+    _gpu(o, "o", torch.float32)
+    _gpu(gate_rows, "gate_rows", torch.float32)
+    _need(gate_rows.shape[0] == T and 0 <= gate_col and gate_col + n <= gate_rows.shape[1], "the gate's columns lie outside its rows")
+    _gpu(weight, "weight", torch.float32, (n,))
+    y = torch.empty(T, n, dtype=out_dtype, device=o.device)
+    gate = ctypes.c_void_p(gate_rows.data_ptr() + 4 * gate_col)
+    _check(state_mixers_lib().ni_gated_rmsnorm(_ptr(o), gate, gate_rows.shape[1], _ptr(weight), _ptr(y), T, n, _float(eps),
+                                               _float(out_scale), dtype_code(out_dtype), _stream()), "gated_rmsnorm")
+    return y
+
+
+def conv_silu(xz: torch.Tensor, inner: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, tail_off: int,
+              seq_of_token: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, state_slot: torch.Tensor,
+              out_dtype: torch.dtype):
+    """``u[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - (taps - 1 - j), c])`` over the first ``inner`` columns of
+    ``xz`` float32 [T, wide], the inputs before a portion's first row taken from the state's tail (per slot, from
+    float ``tail_off`` on: [(taps - 1)][inner], the oldest first), which this call moves on.  Returns ``(u as
+    float32, u in out_dtype)`` (the same tensor when ``out_dtype`` is float32)."""
+    T, wide = xz.shape
+    _gpu(xz, "xz", torch.float32)
+    taps = weight.shape[1]
+    _gpu(weight, "weight", torch.float32, (inner, taps))
+    if bias is not None:
+        _gpu(bias, "bias", torch.float32, (inner,))
+    _need(inner <= wide, "more channels than the rows have")
+    stride = _state(state)
+    _need(stride >= tail_off + (taps - 1) * inner, "the state is too small")
+    _gpu(seq_of_token, "seq_of_token", torch.int32, (T,))
+    B = _per_seq(q_start, q_len, state_slot)
+    u32 = torch.empty(T, inner, dtype=torch.float32, device=xz.device)
+    uc = None if out_dtype == torch.float32 else torch.empty(T, inner, dtype=out_dtype, device=xz.device)
+    _check(state_mixers_lib().ni_conv_silu(_ptr(xz), wide, _ptr(weight), _ptr(bias), _ptr(state), _size_t(stride), _size_t(tail_off),
+                                           _ptr(seq_of_token), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(u32), _ptr(uc),
+                                           T, B, inner, taps, dtype_code(out_dtype), _stream()), "conv_silu")
+    return u32, (u32 if uc is None else uc)
+
+
+def selective_scan(dt_pre: torch.Tensor, dt_bias: torch.Tensor, u: torch.Tensor, xz: torch.Tensor, z_col: int, bc: torch.Tensor,
+                   A: torch.Tensor, D: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                   state_slot: torch.Tensor, N: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """``dt = softplus(dt_pre + dt_bias); S <- exp(dt A) S + dt u B; y = (S . C + D u) * silu(z)`` over the rows of
+    every sequence of the step, in order.  ``dt_pre``, ``u`` float32 [T, inner]; ``z``: the columns ``z_col ..`` of
+    ``xz`` float32 [T, wide]; ``bc`` float32 [T, 2 N]: B | C; ``A`` float32 [inner, n padded] as
+    :func:`scan_state_floats` lays a channel out (negative, padding zero); ``state`` float32 [slots, >=
+    scan_state_floats(inner, N)], moved on.  Returns y [T, inner] in ``out_dtype``."""
+    T, inner = u.shape
+    _gpu(u, "u", torch.float32)
+    _gpu(dt_pre, "dt_pre", torch.float32, (T, inner))
+    _gpu(dt_bias, "dt_bias", torch.float32, (inner,))
+    _gpu(D, "D", torch.float32, (inner,))
+    _gpu(xz, "xz", torch.float32)
+    _need(xz.shape[0] == T and 0 <= z_col and z_col + inner <= xz.shape[1], "the gate's columns lie outside its rows")
+    _gpu(bc, "bc", torch.float32, (T, 2 * N))
+    floats = scan_state_floats(inner, N)
+    _gpu(A, "A", torch.float32, (inner, floats // inner))
+    stride = _state(state)
+    _need(stride >= floats, "the state is too small")
+    B = _per_seq(q_start, q_len, state_slot)
+    y = torch.empty(T, inner, dtype=out_dtype, device=u.device)
+    z = ctypes.c_void_p(xz.data_ptr() + 4 * z_col)
+    _check(state_mixers_lib().ni_selective_scan(_ptr(dt_pre), _ptr(dt_bias), _ptr(u), z, xz.shape[1], _ptr(bc), 2 * N, _ptr(A),
+                                                _ptr(D), _ptr(state), _size_t(stride), _ptr(q_start), _ptr(q_len), _ptr(state_slot),
+                                                _ptr(y), T, B, inner, N, dtype_code(out_dtype), _stream()), "selective_scan")
+    return y

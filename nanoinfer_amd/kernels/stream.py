@@ -59,6 +59,43 @@ def add_vector(h: torch.Tensor, vec: torch.Tensor) -> torch.Tensor:
     return h
 
 
+def embed_pair_hash(ids: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor,
+                    q_len: torch.Tensor, state_slot: torch.Tensor, last_token: torch.Tensor, table: torch.Tensor,
+                    pairs: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int, scale: float, out: torch.Tensor) -> torch.Tensor:
+    """``out[t] = table[ids[t]] * scale + pairs[(prev * mul_prev + ids[t] * mul_cur) mod buckets]`` as float32, ``prev``
+    the token before ``ids[t]`` in its sequence; a sequence's first token (position 0) takes row ``buckets``.
+    ``last_token`` int32 [slots, 1] holds, per state slot, the last token of the sequence so far: it serves the first
+    row of a portion and is moved on by this call."""
+    T = ids.shape[0]
+    B = q_start.shape[0]
+    vocab, d = table.shape
+    for name, t in (("ids", ids), ("positions", positions), ("seq_of_token", seq_of_token)):
+        _gpu(t, name, torch.int32, (T,))
+    for name, t in (("q_start", q_start), ("q_len", q_len), ("state_slot", state_slot)):
+        _gpu(t, name, torch.int32, (B,))
+    _need(last_token.is_cuda and last_token.dtype == torch.int32 and last_token.is_contiguous() and last_token.dim() == 2
+          and last_token.shape[1] == 1, "last_token must be int32 [slots, 1] on the GPU")
+    _gpu(table, "table")
+    _gpu(pairs, "pairs", table.dtype, (buckets + 1, d))
+    _gpu(out, "out", torch.float32, (T, d))
+    _check(stream_lib().ni_embed_pair_hash(_ptr(ids), _ptr(positions), _ptr(seq_of_token), _ptr(q_start), _ptr(q_len),
+                                           _ptr(state_slot), _ptr(last_token), _ptr(table), _ptr(pairs), _ptr(out), T, B, d, vocab,
+                                           int(buckets), ctypes.c_longlong(mul_prev), ctypes.c_longlong(mul_cur), _float(scale),
+                                           dtype_code(table.dtype), _stream()), "embed_pair_hash")
+    return out
+
+
+def add_rows_vector(h: torch.Tensor, extra: Optional[torch.Tensor], vec: torch.Tensor) -> torch.Tensor:
+    """``h[t] = (h[t] + extra[t]) + vec`` for every row of the float32 stream (``extra`` may be absent)."""
+    T, d = h.shape
+    _gpu(h, "h", torch.float32)
+    if extra is not None:
+        _gpu(extra, "extra", torch.float32, (T, d))
+    _gpu(vec, "vec", torch.float32, (d,))
+    _check(stream_lib().ni_add_rows_vector(_ptr(h), _ptr(extra), _ptr(vec), T, d, _stream()), "add_rows_vector")
+    return h
+
+
 def stream_add(h: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None,
                x_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``h += (a + b)`` in float32 (``b`` may be absent); ``x_out``, if given, takes the new stream in its own
@@ -102,28 +139,36 @@ def add_rmsnormed(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: f
 
 # ------------------------------------------------------------------ router and experts
 
-def route_top(z: torch.Tensor, top: int, mix_all: bool):
-    """The ``top`` largest logits of every row of ``z`` float32 [T, E] and their softmax among themselves:
+def route_top(z: torch.Tensor, top: int, mix_all: bool, over_all: bool = False, groups: int = 1, keep: int = 1):
+    """The ``top`` largest logits of every row of ``z`` float32 [T, E] and their weights: the softmax among the
+    chosen, or (``over_all``) the softmax over all E experts, not renormalised.  With ``groups`` > 1 the experts
+    form that many equal groups of neighbours, a group counts as much as its largest logit, and only experts of the
+    ``keep`` best groups can be chosen.
     ``(chosen int32 [T, top], mix float32 [T, top], mix over all experts float32 [T, E] or None)``."""
     T, E = z.shape
     _gpu(z, "z", torch.float32)
     _need(1 <= top <= E, f"{top} of {E} experts cannot be chosen")
+    _need(1 <= groups <= 64 and E % groups == 0 and 1 <= keep <= groups and top <= E // groups * keep,
+          f"{top} experts cannot be chosen from {keep} of {groups} groups of {E} experts")
     chosen = torch.empty(T, top, dtype=torch.int32, device=z.device)
     mix = torch.empty(T, top, dtype=torch.float32, device=z.device)
     dense = torch.empty(T, E, dtype=torch.float32, device=z.device) if mix_all else None
-    _check(stream_lib().ni_route_top(_ptr(z), _ptr(chosen), _ptr(mix), _ptr(dense), T, E, top, _stream()), "route_top")
+    _check(stream_lib().ni_route_top(_ptr(z), _ptr(chosen), _ptr(mix), _ptr(dense), T, E, top, int(bool(over_all)),
+                                     int(groups), int(keep), _stream()), "route_top")
     return chosen, mix, dense
 
 
-def experts_act(up: torch.Tensor, mix_all: torch.Tensor, ff: int) -> torch.Tensor:
-    """``mix_all[t, e] * relu(up[t, e * ff + i])^2`` in the type of ``up``."""
+def experts_act(up: torch.Tensor, mix_all: torch.Tensor, ff: int, gated: bool = False) -> torch.Tensor:
+    """``mix_all[t, e] * relu(up[t, e * ff + i])^2`` in the type of ``up``; ``gated``: an expert's columns of ``up``
+    are [gate: ff | up: ff] and the result is ``mix_all[t, e] * silu(gate) * up``, [T, E * ff]."""
     T, width = up.shape
     E = mix_all.shape[1]
     _gpu(up, "up")
     _gpu(mix_all, "mix_all", torch.float32, (T, E))
-    _need(width == E * ff, "the experts' hidden rows do not match the router")
-    act = torch.empty_like(up)
-    _check(stream_lib().ni_experts_act(_ptr(up), _ptr(mix_all), _ptr(act), T, E, ff, dtype_code(up.dtype), _stream()), "experts_act")
+    _need(width == E * ff * (2 if gated else 1), "the experts' hidden rows do not match the router")
+    act = torch.empty(T, E * ff, dtype=up.dtype, device=up.device)
+    _check(stream_lib().ni_experts_act(_ptr(up), _ptr(mix_all), _ptr(act), T, E, ff, int(bool(gated)), dtype_code(up.dtype), _stream()),
+           "experts_act")
     return act
 
 
@@ -131,21 +176,26 @@ EXPERTS_FEW_ROWS = 16       # up to here only the chosen experts' matrices are r
 
 
 def experts_few(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor, mix: torch.Tensor,
-                ff: int) -> torch.Tensor:
-    """The weighted sum of the chosen experts for a few rows: ``w_up`` [E * ff, d], ``w_down`` [d, E * ff];
-    returns float32 [T, d]."""
+                ff: int, gated: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The weighted sum of the chosen experts for a few rows: ``w_up`` [E * ff, d] (``gated``: [E * 2 ff, d], an
+    expert's gate rows and then its up rows; the hidden row is then ``silu(gate) * up`` instead of ``relu(up)^2``),
+    ``w_down`` [d, E * ff]; returns float32 [T, d] (``out``, if given)."""
     T, d = x.shape
     top = chosen.shape[1]
-    E = w_up.shape[0] // ff
+    per = ff * (2 if gated else 1)
+    E = w_up.shape[0] // per
     _gpu(x, "x", w_up.dtype)
-    _gpu(w_up, "w_up", None, (E * ff, d))
+    _gpu(w_up, "w_up", None, (E * per, d))
     _gpu(w_down, "w_down", w_up.dtype, (d, E * ff))
     _gpu(chosen, "chosen", torch.int32, (T, top))
     _gpu(mix, "mix", torch.float32, (T, top))
     hid = torch.empty(T * top, ff, dtype=torch.float32, device=x.device)
-    out = torch.empty(T, d, dtype=torch.float32, device=x.device)
+    if out is None:
+        out = torch.empty(T, d, dtype=torch.float32, device=x.device)
+    else:
+        _gpu(out, "out", torch.float32, (T, d))
     _check(stream_lib().ni_experts_few(_ptr(x), _ptr(w_up), _ptr(w_down), _ptr(chosen), _ptr(mix), _ptr(hid), _ptr(out),
-                                       T, d, ff, E, top, dtype_code(x.dtype), _stream()), "experts_few")
+                                       T, d, ff, E, top, int(bool(gated)), dtype_code(x.dtype), _stream()), "experts_few")
     return out
 
 
@@ -246,17 +296,54 @@ def kv_store(qkv: torch.Tensor, k_off: int, v_off: int, slot_mapping: torch.Tens
                                             T, G, dk, dv, ps, dtype_code(qkv.dtype), _stream()), "kv_store")
 
 
+def qk_norm_rope_store(proj: torch.Tensor, positions: torch.Tensor, slot_mapping: Optional[torch.Tensor],
+                       q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float, freq: Optional[torch.Tensor],
+                       amplitude: float, q_out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, H: int) -> torch.Tensor:
+    """From ``proj`` float32 [T, H*dk + G*dk + G*dv] (q | k | v as projected): the RMS norm over a token's WHOLE
+    query projection and over its whole key projection (weights ``q_norm`` [H*dk], ``k_norm`` [G*dk]; None: no norm),
+    then the rotation of the first ``2 * len(freq)`` channels of every head, channel c with channel c + len(freq), by
+    ``position * freq[c]`` with cos and sin times ``amplitude`` (``freq`` None: no rotation), all in float32.  Queries
+    go to ``q_out`` [T, H*dk], keys and values into their page slots (``slot_mapping`` None: nothing is stored)."""
+    T, width = proj.shape
+    pages, G, ps, dk = kpool.shape
+    dv = vpool.shape[3]
+    _gpu(proj, "proj", torch.float32)
+    _need(width == (H + G) * dk + G * dv, "proj is not q | k | v of these sizes")
+    _gpu(positions, "positions", torch.int32, (T,))
+    if slot_mapping is not None:
+        _gpu(slot_mapping, "slot_mapping", torch.int32, (T,))
+    if q_norm is not None:
+        _gpu(q_norm, "q_norm", torch.float32, (H * dk,))
+    if k_norm is not None:
+        _gpu(k_norm, "k_norm", torch.float32, (G * dk,))
+    rot = 0
+    if freq is not None:
+        rot = 2 * freq.shape[0]
+        _gpu(freq, "freq", torch.float32, (rot // 2,))
+        _need(0 < rot <= dk, f"{rot} rotated channels do not fit a head of {dk}")
+    _gpu(kpool, "kpool")
+    _gpu(vpool, "vpool", kpool.dtype, (pages, G, ps, dv))
+    _gpu(q_out, "q_out", kpool.dtype, (T, H * dk))
+    _check(bias_attention_lib().ni_qk_norm_rope_store(_ptr(proj), width, _ptr(positions), _ptr(slot_mapping), _ptr(q_norm),
+                                                      _ptr(k_norm), _float(eps), _ptr(freq), rot, _float(amplitude), _ptr(q_out),
+                                                      _ptr(kpool), _ptr(vpool), T, H, G, dk, dv, ps, dtype_code(kpool.dtype),
+                                                      _stream()), "qk_norm_rope_store")
+    return q_out
+
+
 def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int, scale: float,
                    temp_coef: float, temp_every: int, heads_per_chunk: int, n_runs: int = 1,
-                   workspace: Optional[torch.Tensor] = None, waves: int = 4) -> torch.Tensor:
+                   workspace: Optional[torch.Tensor] = None, waves: int = 4, window: Optional[int] = None, keep_first: int = 0,
+                   out_scale: float = 1.0) -> torch.Tensor:
     """Causal attention of the query heads in the first ``H * dk`` columns of ``qkv`` over the paged cache.
     ``tiles`` int32 [n, 4]: (sequence, first row, tokens, -) with tokens * heads of a chunk <= 16, the tokens of a
     tile being consecutive ones of one sequence; ``positions`` int32 [T] the position of every row;
     ``bias`` float32 [distances, H] or None; ``out`` [T, H * dv].  With ``n_runs`` > 1 the keys of every tile are
     cut into that many runs, which meet in ``workspace`` (float32, at least T * H * n_runs * (dv + 2)) and are merged
     by a second kernel.  ``waves`` (1 to 4): wavefronts of a workgroup, four rows each; fewer than four only where no
-    tile has more rows than they take."""
+    tile has more rows than they take.  ``window`` n: a query sees its last n keys (its own among them) and the first
+    ``keep_first`` keys of its sequence; ``out_scale`` multiplies the output."""
     T, width = qkv.shape
     pages, G, ps, dk = kpool.shape
     dv = vpool.shape[3]
@@ -286,6 +373,7 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
                                                  block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions), _ptr(bias), distances,
                                                  _ptr(out), H, G, dk, dv, ps, _float(scale), _float(temp_coef), int(temp_every),
                                                  heads_per_chunk, n_runs, _ptr(workspace if n_runs > 1 else None), T, waves,
+                                                 int(window or 0), int(keep_first), _float(out_scale),
                                                  dtype_code(qkv.dtype), _stream())
     if err == -2:
         raise KernelError(f"keys of {dk} and values of {dv} channels do not fit the kernel's staging memory")
@@ -304,7 +392,8 @@ def bias_attention_mfma_rows(dk: int, dv: int) -> int:
 
 def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                         tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int,
-                        scale: float, temp_coef: float, temp_every: int, heads_per_chunk: int) -> torch.Tensor:
+                        scale: float, temp_coef: float, temp_every: int, heads_per_chunk: int, window: Optional[int] = None,
+                        keep_first: int = 0, out_scale: float = 1.0) -> torch.Tensor:
     """:func:`bias_attention` for steps with portions of prompts: tiles of up to 64 rows (tokens * heads of a chunk),
     both products on the float32 matrix instructions, the same formula and the same 32-bit softmax; no runs."""
     T, width = qkv.shape
@@ -331,5 +420,6 @@ def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Ten
                                                        block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions),
                                                        _ptr(bias), distances, _ptr(out), H, G, dk, dv, ps, _float(scale),
                                                        _float(temp_coef), int(temp_every), heads_per_chunk,
+                                                       int(window or 0), int(keep_first), _float(out_scale),
                                                        dtype_code(qkv.dtype), _stream()), "bias_attention_mfma")
     return out

@@ -75,7 +75,9 @@ class ScaledTableEmbedding(Part):
 @register_part("pass_input", "vector_rows")
 class VectorRows(Part):
     """A table of learned vectors, one of which is added to every row of the stream where an entry of the
-    order says so (``LayerRun.enter``).  params: rows, size.  weights: table [rows, size]."""
+    order says so (``LayerRun.enter``).  params: rows, size, again (default False: with it, every pass but the
+    first also adds the embedding's output, the stream as it was before the first layer, ahead of the vector).
+    weights: table [rows, size]."""
 
     graph_safe = True
 
@@ -87,12 +89,18 @@ class VectorRows(Part):
         super().__init__(spec, weights, rt)
         table = weights["table"].to(device=rt.device, dtype=torch.float32).contiguous()
         self.rows = [table[i] for i in range(table.shape[0])]
+        # the model keeps a copy of the embedding's output for a pass input that says so, and hands it to forward
+        self.wants_embedding = bool(spec.params.get("again", False)) and len(self.rows) > 1
 
     def settle(self, h: torch.Tensor, pending: Optional[torch.Tensor]) -> torch.Tensor:
         """``h`` with an addend it has not received yet."""
         return h if pending is None else K.stream_add(h, pending.contiguous())
 
-    def forward(self, h: torch.Tensor, row: int) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, row: int, embedded: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if self.wants_embedding:
+            if embedded is None:
+                raise K.KernelError("this pass input adds the embedding's output again and was not given it")
+            return K.add_rows_vector(h, embedded if row > 0 else None, self.rows[row])
         return K.add_vector(h, self.rows[row])
 
 
@@ -206,18 +214,23 @@ class BiasAttention(Part):
         return CacheNeed(kv=KVNeed(self.G, self.dk, None, self.dv))
 
     def forward(self, x, ctx, cache: LayerCache):
-        T = x.shape[0]
         qkv = K.linear(x, self.w_qkv)
         if cache.writes:
             K.kv_store(qkv, self.H * self.dk, (self.H + self.G) * self.dk, cache.slot_mapping, cache.kpool, cache.vpool)
+        return K.linear(self.attend(qkv, ctx, cache), self.w_o, out_dtype=torch.float32)
+
+    def attend(self, qkv, ctx, cache: LayerCache, window: Optional[int] = None, keep_first: int = 0, out_scale: float = 1.0):
+        """The queries in the first ``H * dk`` columns of ``qkv`` over the keys and values of the cache: [T, H * dv] in
+        the compute type.  ``window`` n: a query sees its last n keys and the sequence's first ``keep_first``;
+        ``out_scale`` multiplies the result."""
+        T = qkv.shape[0]
         out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
         if self.wide_heads and ctx.max_q_len >= K.BIAS_ATTENTION_MFMA_FROM:
             tiles = ctx.q_tiles(self.wide_tokens)
             if tiles is None:
                 raise K.KernelError("this step was recorded without the tiles of its tokens")
-            K.bias_attention_mfma(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H,
-                                  self.scale, self.temp_coef, self.temp_every, self.wide_heads)
-            return K.linear(out, self.w_o, out_dtype=torch.float32)
+            return K.bias_attention_mfma(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H,
+                                         self.scale, self.temp_coef, self.temp_every, self.wide_heads, window, keep_first, out_scale)
         tiles = ctx.q_tiles(self.tile_tokens)
         if tiles is None:
             raise K.KernelError("this step was recorded without the tiles of its tokens")
@@ -227,11 +240,13 @@ class BiasAttention(Part):
         # all four wavefronts stage the keys and values, also where fewer of them have rows; the keys are cut into
         # runs by the wavefronts that have rows
         waves = 4
-        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, ctx.max_context, min(4, -(-rows // 4)))
+        # with a window a tile walks the kept first keys, the window and its own tokens, in whole tiles of 64 keys
+        max_keys = ctx.max_context if window is None else min(ctx.max_context, window + keep_first + self.tile_tokens + 128)
+        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, max_keys, min(4, -(-rows // 4)))
         ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
-        K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H, self.scale,
-                         self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves)
-        return K.linear(out, self.w_o, out_dtype=torch.float32)
+        return K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H,
+                                self.scale, self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves, window,
+                                keep_first, out_scale)
 
 
 # ------------------------------------------------------------------ gated delta rule, a decay per key channel
@@ -326,14 +341,22 @@ class ChannelDelta(Part):
 
 @register_part("feed_forward", "routed_experts")
 class RoutedExperts(Part):
-    """``experts`` small feed-forwards ``W_down act(W_up x)`` of which every token uses the ``top`` with the
-    largest router logits ``W_r x`` (float32), mixed by the softmax over the chosen logits alone.
-    params: hidden_size, expert_size, experts, top, activation ("relu2": the square of relu).
-    weights: router [experts, d], up<e> [expert_size, d], down<e> [d, expert_size].
+    """``experts`` small feed-forwards of which every token uses the ``top`` with the largest router logits
+    ``W_r x`` (float32), and optionally one more (``shared``) that every token uses with weight 1.
 
-    The experts' matrices are laid side by side, up [E * ff, d] and down [d, E * ff].  For a few rows only
-    the chosen experts' rows are read; for many, all experts run as two dense products with the mix of an
-    expert that was not chosen at zero, which the matrix cores do faster than a gather would here."""
+    params: hidden_size, expert_size, experts, top;
+    activation: "relu2" (an expert is ``W_down relu(W_up x)^2``) or "swiglu" (``W_down (silu(W_gate x) * (W_up x))``);
+    mix: "softmax_chosen" (the softmax over the chosen logits alone, the default) or "softmax_all" (the softmax over all
+    experts, the chosen ones' shares not renormalised); groups, keep (default 1, 1): the experts form ``groups`` equal
+    groups of neighbours, a group counts as much as its best expert, and only the best ``keep`` groups can be chosen from;
+    shared: None or the PartSpec of a feed-forward.
+    weights: router [experts, d], up<e> [expert_size, d], down<e> [d, expert_size], with "swiglu" also gate<e>.
+
+    The experts' matrices are laid side by side, up [E * ff, d] (gated: [E * 2 ff, d], an expert's gate rows and then
+    its up rows) and down [d, E * ff].  For a few rows only the chosen experts' rows are read; for many, all experts
+    run as two dense products with the mix of an expert that was not chosen at zero, which the matrix cores do
+    faster than a gather would here.  With a shared expert the result is two float32 addends [2, T, d], which the
+    next norm sums in float32."""
 
     graph_safe = True
 
@@ -343,30 +366,55 @@ class RoutedExperts(Part):
         d, ff = p["hidden_size"], p["expert_size"]
         out = [WeightRequest(w["router"], (p["experts"], d))]
         for e in range(p["experts"]):
+            if p.get("activation", "relu2") == "swiglu":
+                out.append(WeightRequest(w[f"gate{e}"], (ff, d)))
             out += [WeightRequest(w[f"up{e}"], (ff, d)), WeightRequest(w[f"down{e}"], (d, ff))]
+        if p.get("shared") is not None:
+            from .standard import requests_of
+            out += requests_of("feed_forward", p["shared"])
         return out
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         p, names = spec.params, spec.weights
         self.E, self.top, self.ff = int(p["experts"]), int(p["top"]), int(p["expert_size"])
-        if p.get("activation", "relu2") != "relu2":
-            raise ValueError(f"expert activation {p['activation']!r} is not known (known: 'relu2')")
+        activation = p.get("activation", "relu2")
+        if activation not in ("relu2", "swiglu"):
+            raise ValueError(f"expert activation {activation!r} is not known (known: 'relu2', 'swiglu')")
+        self.gated = activation == "swiglu"
+        mix = p.get("mix", "softmax_chosen")
+        if mix not in ("softmax_chosen", "softmax_all"):
+            raise ValueError(f"expert mix {mix!r} is not known (known: 'softmax_chosen', 'softmax_all')")
+        self.over_all = mix == "softmax_all"
+        self.groups, self.keep = int(p.get("groups", 1)), int(p.get("keep", 1))
+        if self.groups < 1 or self.E % self.groups or not 1 <= self.keep <= self.groups or self.top > self.E // self.groups * self.keep:
+            raise ValueError(f"{self.top} experts cannot be chosen from {self.keep} of {self.groups} groups of {self.E}")
         self.w_router = rt.weight(names["router"], weights["router"])
-        self.w_up = rt.weight("|".join(names[f"up{e}"] for e in range(self.E)),
-                              torch.cat([weights[f"up{e}"] for e in range(self.E)], dim=0), tiled=False)
+        order = [k for e in range(self.E) for k in ((f"gate{e}", f"up{e}") if self.gated else (f"up{e}",))]
+        self.w_up = rt.weight("|".join(names[k] for k in order), torch.cat([weights[k] for k in order], dim=0), tiled=False)
         self.w_down = rt.weight("|".join(names[f"down{e}"] for e in range(self.E)),
                                 torch.cat([weights[f"down{e}"] for e in range(self.E)], dim=1), tiled=False)
+        self.shared = None
+        if p.get("shared") is not None:
+            self.shared = build_part("feed_forward", p["shared"], getattr(weights, "checkpoint", {}), rt)
 
     def forward(self, x, ctx):
         T = x.shape[0]
         z = K.linear(x, self.w_router, out_dtype=torch.float32)
         few = T <= K.EXPERTS_FEW_ROWS
-        chosen, mix, mix_all = K.route_top(z, self.top, mix_all=not few)
+        chosen, mix, mix_all = K.route_top(z, self.top, mix_all=not few, over_all=self.over_all, groups=self.groups, keep=self.keep)
+        out = None
+        if self.shared is not None:
+            out = torch.empty(2, T, self.w_down.shape[0], dtype=torch.float32, device=x.device)
         if few:
-            return K.experts_few(x, self.w_up.rows, self.w_down.rows, chosen, mix, self.ff)
-        act = K.experts_act(K.linear(x, self.w_up), mix_all, self.ff)
-        return K.linear(act, self.w_down, out_dtype=torch.float32)
+            y = K.experts_few(x, self.w_up.rows, self.w_down.rows, chosen, mix, self.ff, self.gated, None if out is None else out[0])
+        else:
+            act = K.experts_act(K.linear(x, self.w_up), mix_all, self.ff, self.gated)
+            y = K.linear(act, self.w_down, out_dtype=torch.float32, out=None if out is None else out[0])
+        if out is None:
+            return y
+        K.linear(self.shared.hidden(x), self.shared.w_down, out_dtype=torch.float32, out=out[1])
+        return out
 
 
 # ------------------------------------------------------------------ block

@@ -139,30 +139,57 @@ def llama3_scaling(freqs: np.ndarray, params: dict) -> np.ndarray:
     return out
 
 
-def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[dict]) -> np.ndarray:
+@register_rope_scaling("yarn")
+def yarn_scaling(freqs: np.ndarray, params: dict) -> np.ndarray:
+    """Pairs that turn fewer than ``slow`` times over ``original`` positions are divided by ``factor``, pairs that
+    turn more than ``fast`` times are kept, a linear ramp over the pair index between:
+    ``pair(t) = dims ln(original / (2 pi t)) / (2 ln base)``, ``lo = max(floor(pair(fast)), 0)``,
+    ``hi = min(ceil(pair(slow)), dims - 1)``, ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``,
+    ``f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i)``.  params: factor, original, fast, slow, dims, base.  (What
+    the rule does to cos and sin, a factor ``0.1 ln(factor) + 1``, is the position part's ``amplitude``.)"""
+    dims, base = int(params["dims"]), float(params["base"])
+    factor, original = float(params["factor"]), float(params["original"])
+
+    def pair(turns: float) -> float:
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+    lo = max(math.floor(pair(float(params["fast"]))), 0)
+    hi = min(math.ceil(pair(float(params["slow"]))), dims - 1)
+    ramp = np.clip((np.arange(freqs.shape[0], dtype=np.float64) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    f = freqs.astype(np.float64)
+    return f / factor * ramp + f * (1.0 - ramp)
+
+
+def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[dict], exact: bool = False) -> np.ndarray:
     """Frequency of each rotated pair, ``theta^(-2p/rotary_dim)`` in float32 arithmetic
     (src/op/kernels/cuda/rope_kernel.cu:103-106), then the scaling rule that ``scaling["kind"]``
-    names, if any, applied with the other entries of ``scaling`` as its parameters."""
+    names, if any, applied with the other entries of ``scaling`` as its parameters.  ``exact``: powers and
+    rule in float64, rounded to float32 once at the end."""
     f32 = np.float32
     half = rotary_dim // 2
-    out = np.empty(half, dtype=f32)
-    for p in range(half):
-        out[p] = f32(1.0) / f32(np.power(f32(theta), f32(f32(2 * p) / f32(rotary_dim)), dtype=f32))
+    if exact:
+        out = np.array([float(theta) ** (-2.0 * p / rotary_dim) for p in range(half)], dtype=np.float64)
+    else:
+        out = np.empty(half, dtype=f32)
+        for p in range(half):
+            out[p] = f32(1.0) / f32(np.power(f32(theta), f32(f32(2 * p) / f32(rotary_dim)), dtype=f32))
     if scaling is not None:
         kind = scaling.get("kind")
         if kind not in ROPE_SCALINGS:
             raise ValueError(f"rotation scaling of kind {kind!r} is not registered; known: {sorted(ROPE_SCALINGS)}")
-        out = np.asarray(ROPE_SCALINGS[kind](out, scaling), dtype=f32)
+        out = np.asarray(ROPE_SCALINGS[kind](out, scaling))
         if out.shape != (half,):
             raise ValueError(f"rotation scaling {kind!r} returned {out.shape} frequencies for {half} pairs")
-    return out
+    return np.asarray(out, dtype=f32)
 
 
 @register_part("position", "rope")
 class RotaryPosition(Part):
     """Rotation of pairs by ``pos * f_p``.  params: rotary_dim, theta, max_positions, scaling (None,
     or a dict with the ``kind`` of a registered rule and that rule's parameters).  One table per
-    distinct set of constants is shared by all layers."""
+    distinct set of constants is shared by all layers.  With ``max_positions`` None (a design without a last
+    position) there is no table: the mixer takes :meth:`frequencies` and works the angles out itself.
+    ``amplitude`` (default 1) is a factor on cos and sin; ``exact``: the frequencies are worked out in float64."""
 
     graph_safe = True
 
@@ -170,19 +197,27 @@ class RotaryPosition(Part):
         super().__init__(spec, weights, rt)
         p = spec.params
         self.rotary_dim = int(p["rotary_dim"])
-        self.max_positions = int(p["max_positions"])
+        self.max_positions = None if p.get("max_positions") is None else int(p["max_positions"])
+        self.amplitude = float(p.get("amplitude", 1.0))
         if self.rotary_dim % 2 or self.rotary_dim <= 0:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be positive and even")
         scaling = p.get("scaling")
-        key = ("rope", self.rotary_dim, float(p["theta"]), self.max_positions,
+        key = ("rope", self.rotary_dim, float(p["theta"]), self.max_positions, bool(p.get("exact", False)),
                None if scaling is None else tuple(sorted(scaling.items())))
         if key not in rt.shared:
-            inv = torch.from_numpy(rope_inverse_frequencies(self.rotary_dim, float(p["theta"]), scaling)).to(rt.device)
-            rt.shared[key] = K.rope_table(inv, self.max_positions)
-        self.cos, self.sin = rt.shared[key]
+            inv = torch.from_numpy(rope_inverse_frequencies(self.rotary_dim, float(p["theta"]), scaling,
+                                                            exact=bool(p.get("exact", False)))).to(rt.device)
+            rt.shared[key] = (inv,) + ((None, None) if self.max_positions is None else tuple(K.rope_table(inv, self.max_positions)))
+        self.inv_freq, self.cos, self.sin = rt.shared[key]
+        if self.cos is not None and self.amplitude != 1.0:
+            raise ValueError("a rotation table with an amplitude is not built; leave max_positions out")
 
     def tables(self):
-        return self.cos, self.sin
+        return None if self.cos is None else (self.cos, self.sin)
+
+    def frequencies(self):
+        """(float32 [rotary_dim / 2] on the device, factor on cos and sin)."""
+        return self.inv_freq, self.amplitude
 
 
 @register_part("position", "none")
@@ -426,11 +461,15 @@ class SwiGLU(Part):
     def leaves_scaled(self, T: int) -> bool:
         return self.adds_residual(T) and K.leaves_scaled_ok(T, self.intermediate_size, self.rt.dtype, self.w_down)
 
+    def hidden(self, x) -> torch.Tensor:
+        """``silu(W_gate x) * (W_up x)``: what the down product takes (for a part that places that product's result itself)."""
+        return K.linear_swiglu(x, self.w_gate_up)
+
     def forward(self, x, ctx, residual: Optional[torch.Tensor] = None, leave=None):
         carried = getattr(x, "pending", None)       # addends of the residual stream that came with a normed input
         if carried is not None and residual is None:
             raise K.KernelError("pending addends of the residual stream need residual=h to go into")
-        return K.linear(K.linear_swiglu(x, self.w_gate_up), self.w_down, residual=residual, pending=carried, leave=leave)
+        return K.linear(self.hidden(x), self.w_down, residual=residual, pending=carried, leave=leave)
 
 
 # ------------------------------------------------------------------ block
@@ -452,6 +491,18 @@ class PreNormBlock(Block):
     """
 
     ROLES = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
+    OPTIONAL = ("ffn_norm", "ffn")      # a block without a feed-forward: ``h += mixer(norm1(h))`` alone
+
+    @classmethod
+    def _roles(cls, spec):
+        missing = [r for r in cls.ROLES if r not in spec.parts and r not in cls.OPTIONAL]
+        extra = [r for r in spec.parts if r not in cls.ROLES]
+        if ("ffn" in spec.parts) != ("ffn_norm" in spec.parts):
+            missing.append("ffn_norm" if "ffn" in spec.parts else "ffn")
+        if missing or extra:
+            raise ValueError(f"a block of kind {spec.kind!r} has the parts {sorted(cls.ROLES)}; "
+                             f"missing: {missing}, not known: {extra}")
+        return [(r, f) for r, f in cls.ROLES.items() if r in spec.parts]
 
     def _normed_input(self, norm, part, h, pending):
         """What ``part`` is given for ``norm(h + pending)``: the norm as a prologue where both sides can, else its
@@ -498,12 +549,14 @@ class PreNormBlock(Block):
     def forward(self, h, pending, ctx, cache: LayerCache, leave=None):
         T = h.shape[0]
         x = self._normed_input(self.mixer_norm, self.mixer, h, pending)
+        if "ffn" not in self.roles:
+            return h, self._addend(self.mixer.forward(x, ctx, cache))
         adds = getattr(self.mixer, "adds_residual", None)
         if adds is not None and adds(T):
             spec = self._deferred(self.ffn_norm, self.mixer, self.ffn, T)
             a = self.mixer.forward(x, ctx, cache, residual=h, **({} if spec is None else {"leave": spec}))
         else:
-            a = self.mixer.forward(x, ctx, cache)
+            a = self._addend(self.mixer.forward(x, ctx, cache))
         x = self._normed_input(self.ffn_norm, self.ffn, h, a)
         adds = getattr(self.ffn, "adds_residual", None)
         if adds is not None and adds(T):
@@ -511,8 +564,15 @@ class PreNormBlock(Block):
             spec = leave if (leave is not None and leaves is not None and leaves(T)) else None
             f = self.ffn.forward(x, ctx, residual=h, **({} if spec is None else {"leave": spec}))
         else:
-            f = self.ffn.forward(x, ctx)
+            f = self._addend(self.ffn.forward(x, ctx))
         return h, f
+
+    def _addend(self, y):
+        """What a part returned, as the next norm takes it: a float32 result [T, d] of a part that keeps its
+        product's accumulators counts as one float32 addend [1, T, d] where the compute type is narrower."""
+        if isinstance(y, torch.Tensor) and y.dim() == 2 and y.dtype == torch.float32 and self.rt.dtype != torch.float32:
+            return y.unsqueeze(0)
+        return y
 
 
 # ------------------------------------------------------------------ head
