@@ -100,9 +100,10 @@ def window_attention(h: np.ndarray, m: dict, w: Dict[str, np.ndarray], pre: str,
     k = rms(h @ w[pre + "k"].T, eps) * w[pre + "k.norm"]
     v = (h @ w[pre + "v"].T).reshape(T, G, dv)
     pos = np.arange(T)
-    q = rotate(q.reshape(T, H, dk), pos, m["rot"])
-    k = rotate(k.reshape(T, G, dk), pos, m["rot"])
-    size, keep = m["mask"]["size"], m["mask"]["keep_first"]
+    q, k = q.reshape(T, H, dk), k.reshape(T, G, dk)
+    if m.get("rot") is not None:
+        q, k = rotate(q, pos, m["rot"]), rotate(k, pos, m["rot"])
+    size, keep = (m["mask"]["size"], m["mask"].get("keep_first", 0)) if m.get("mask") is not None else (T + 1, 0)
     out = np.zeros((T, H, dv), dtype=F)
     for hd in range(H):
         g = hd // (H // G)
@@ -167,30 +168,43 @@ def gated_ff(h, w, pre):
 
 
 def route(z: np.ndarray, router: dict):
-    """For one token's router logits: (chosen experts, their weights)."""
+    """For one token's router logits: (chosen experts, their weights, how close the closest call was: the smallest
+    difference of logits between something chosen and something left out, a group or an expert)."""
     E, top = router["experts"], router["top"]
     s = np.exp(z - z.max())
     s = s / s.sum()
     allowed = np.ones(E, dtype=bool)
     groups = router.get("groups")
+    margin = np.inf
     if groups is not None:
         n = groups["count"]
         per = E // n
-        best = np.argsort(-s.reshape(n, per).max(axis=1), kind="stable")[: groups["keep"]]
+        score = s.reshape(n, per).max(axis=1)
+        ranked = np.argsort(-score, kind="stable")
+        best = ranked[: groups["keep"]]
+        if groups["keep"] < n:
+            top_logit = z.reshape(n, per).max(axis=1)
+            margin = top_logit[ranked[groups["keep"] - 1]] - top_logit[ranked[groups["keep"]]]
         allowed[:] = False
         for g in best:
             allowed[g * per: (g + 1) * per] = True
-    order = np.argsort(-np.where(allowed, s, -1.0), kind="stable")[:top]
-    return order, s[order]
+    ranked = np.argsort(-np.where(allowed, s, -1.0), kind="stable")
+    order = ranked[:top]
+    if top < int(allowed.sum()):
+        margin = min(margin, z[ranked[top - 1]] - z[ranked[top]])
+    return order, s[order], margin
 
 
-def moe(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str) -> np.ndarray:
+def moe(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str, margins: Optional[list] = None) -> np.ndarray:
     out = np.zeros_like(h)
     z = h @ w[pre + "router"].T
+    closest = np.full(h.shape[0], np.inf)
     for t in range(h.shape[0]):
-        chosen, weight = route(z[t], mlp["router"])
+        chosen, weight, closest[t] = route(z[t], mlp["router"])
         for e, a in zip(chosen, weight):
             out[t] += a * gated_ff(h[t: t + 1], w, f"{pre}e{e}.")[0]
+    if margins is not None:
+        margins.append(closest)
     if mlp.get("shared") is not None:
         out += gated_ff(h, w, pre + "shared.")
     return out
@@ -198,7 +212,7 @@ def moe(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str) -> np.ndar
 
 # ------------------------------------------------------------------ the model
 
-def layer(x, i: int, cfg: dict, w):
+def layer(x, i: int, cfg: dict, w, margins: Optional[list] = None):
     L = cfg["layers"][i]
     eps = cfg["norm"]["eps"]
     pre = f"l{i}."
@@ -210,7 +224,7 @@ def layer(x, i: int, cfg: dict, w):
     else:
         raise ValueError(L["type"])
     if L.get("mlp") is not None:
-        x = x + moe(rms(x, eps) * w[pre + "norm2"], L["mlp"], w, pre + "mlp.")
+        x = x + moe(rms(x, eps) * w[pre + "norm2"], L["mlp"], w, pre + "mlp.", margins)
     return x
 
 
@@ -226,8 +240,10 @@ def layer_runs(cfg: dict):
     return runs + [(i, None) for i in range(lp["stop"], L)]
 
 
-def forward(tokens: List[int], cfg: dict, weights: Dict[str, np.ndarray], taps: Optional[list] = None) -> np.ndarray:
-    """Logits [T, vocab] of one whole sequence; ``taps`` (a list) receives the stream after every layer run."""
+def forward(tokens: List[int], cfg: dict, weights: Dict[str, np.ndarray], taps: Optional[list] = None,
+            margins: Optional[list] = None) -> np.ndarray:
+    """Logits [T, vocab] of one whole sequence; ``taps`` (a list) receives the stream after every layer run,
+    ``margins`` (a list) per routed layer run the closest call of its router for every token."""
     w = {k: np.asarray(v, dtype=F) for k, v in weights.items()}
     e = embed(tokens, cfg, w)
     x = e.copy()
@@ -236,8 +252,41 @@ def forward(tokens: List[int], cfg: dict, weights: Dict[str, np.ndarray], taps: 
             if enters > 0:
                 x = x + e
             x = x + w["loop.step"][enters]
-        x = layer(x, i, cfg, w)
+        x = layer(x, i, cfg, w, margins)
         if taps is not None:
             taps.append(x.copy())
     x = rms(x, cfg["norm"]["eps"]) * w["final.norm"]
     return x @ w["head"].T
+
+
+# ------------------------------------------------------------------ a model folder, read without the engine
+
+def read_model_folder(folder: str):
+    """(config.json as a dict, tensor name -> float64 array) of a folder with ``model.safetensors``: eight bytes of
+    header length, the JSON header (name -> dtype, shape, data_offsets), the data."""
+    import json
+    import os
+    import struct
+    with open(os.path.join(folder, "config.json")) as fh:
+        cfg = json.load(fh)
+    with open(os.path.join(folder, "model.safetensors"), "rb") as fh:
+        blob = fh.read()
+    n = struct.unpack("<Q", blob[:8])[0]
+    header = json.loads(blob[8: 8 + n])
+    data = blob[8 + n:]
+    out = {}
+    for name, info in header.items():
+        if name == "__metadata__":
+            continue
+        a, b = info["data_offsets"]
+        raw = data[a:b]
+        if info["dtype"] == "BF16":
+            arr = (np.frombuffer(raw, dtype="<u2").astype(np.uint32) << 16).view(np.float32)
+        elif info["dtype"] == "F32":
+            arr = np.frombuffer(raw, dtype="<f4")
+        elif info["dtype"] == "I32":
+            arr = np.frombuffer(raw, dtype="<i4")
+        else:
+            raise ValueError(f"{name}: dtype {info['dtype']}")
+        out[name] = arr.astype(F).reshape(info["shape"])
+    return cfg, out

@@ -1,0 +1,658 @@
+"""Fusavik through the engine against the plain implementation (``plain_fusavik.py``): every mechanism alone and
+all together, whole prompts against portions and single tokens, unequal batches against each request alone, pages
+and state slots that are used again, keys far back, at the edges of pages and of the kernel's tiles of 64 keys, and
+just inside and outside the window and the kept first tokens, long decoding, and greedy generation through ``Engine``.
+
+Models are written with the random-weights mode in bfloat16 (so that both compute types see the same numbers as
+the plain implementation) with larger matrices than the architecture's rule draws, so that a mixer or feed-forward
+that went wrong moves the logits by far more than the tolerance; where random weights would still hide a fault (one
+key among hundreds, the window's edge) the test makes the inputs that show it.
+"""
+import functools
+import json
+import os
+import shutil
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+import plain_fusavik as P
+import fusavik_configs as Z
+import gpu_common
+from gpu_common import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+_root = None
+_folders = {}
+
+
+def folder_of(name: str, seed: int = 11) -> str:
+    global _root
+    key = (name, seed)
+    if key not in _folders:
+        import nanoinfer_amd  # noqa: F401
+        from nanoinfer_amd.weights.loader import make_random_model
+        if _root is None:
+            _root = tempfile.mkdtemp(prefix="fusavik-tests-")
+            import atexit
+            atexit.register(shutil.rmtree, _root, ignore_errors=True)
+        _folders[key] = make_random_model(os.path.join(_root, f"{name}-{seed}-{len(_folders)}"), Z.ALL[name], seed,
+                                          dtype="bfloat16", matrix_std=0.12)
+    return _folders[key]
+
+
+_margins = {}      # id of a plain result -> per row, the closest call any router of the model made for it
+
+
+@functools.lru_cache(maxsize=None)
+def _model(folder: str):
+    return P.read_model_folder(folder)
+
+
+@functools.lru_cache(maxsize=None)
+def plain(folder: str, tokens: tuple) -> torch.Tensor:
+    cfg, w = _model(folder)
+    margins = []
+    out = torch.from_numpy(P.forward(list(tokens), cfg, w, margins=margins))
+    if margins:
+        _margins[id(out)] = torch.from_numpy(np.stack(margins).min(axis=0))
+    return out
+
+
+def runner_for(folder, dtype, **kw):
+    from nanoinfer_amd.engine.runner import ModelRunner
+    kw.setdefault("page_size", 8)
+    kw.setdefault("max_tokens", 2048)
+    kw.setdefault("max_requests", 4)
+    return ModelRunner(folder, dtype=dtype, **kw)
+
+
+def replay(runner, requests, steps):
+    """Run ``steps`` (each a dict request -> number of its next tokens), asking for every row; returns
+    request -> logits [tokens, vocab].  A request ends with its last token."""
+    from nanoinfer_amd.engine.runner import StepEntry
+    done = {r: 0 for r in requests}
+    rows = {r: [] for r in requests}
+    for counts in steps:
+        entries = [StepEntry(r, list(requests[r][done[r]:done[r] + c]), list(range(c))) for r, c in counts.items()]
+        out = runner.step(entries, end=[r for r, c in counts.items() if done[r] + c == len(requests[r])])
+        at = 0
+        for r, c in counts.items():
+            rows[r].append(out[at:at + c].clone())
+            at += c
+            done[r] += c
+    assert all(done[r] == len(requests[r]) for r in requests)
+    return {r: torch.cat(v) for r, v in rows.items()}
+
+
+def cuts(n, sizes):
+    out, i = [], 0
+    while n > 0:
+        c = min(n, sizes[i % len(sizes)])
+        out.append(c)
+        n -= c
+        i += 1
+    return out
+
+
+DTYPES = ["float32", "bfloat16"]
+
+# Float32 is the sharp comparison: every row within 2e-5 of its own largest logit.  bfloat16 is judged row by row by
+# the root mean square of the difference over the vocabulary (its mean taken off) against the root mean square of the
+# plain logits; the models are drawn with large matrices on purpose, so rounding weighs more than in a trained model
+# and a close call of a router now and then goes the other way; a token that went to another expert also leaves
+# another trace in the states of the layers behind it, which the later rows of its sequence read.  The median row
+# within 2.5e-2; among the rows before the sequence's first close call (a margin under 0.15 between what was chosen
+# and what was left out) at most one in ten beyond 5e-2 and none beyond 0.3.  A fault (a lost state, a key too many)
+# moves many rows by the size of the logits themselves.
+BF16_MEDIAN, BF16_ROW, BF16_WORST = 2.5e-2, 5e-2, 0.3
+worst_bf16_row = [0.0]
+
+
+def assert_close(got, want, dtype, what=""):
+    if dtype == "float32":
+        return gpu_common.assert_close(got, want, dtype, what)
+    assert tuple(got.shape) == tuple(want.shape), what
+    diff = got.double().cpu() - want
+    diff = diff - diff.mean(dim=-1, keepdim=True)
+    per_row = diff.pow(2).mean(dim=-1).sqrt() / want.pow(2).mean().sqrt()
+    assert float(per_row.median()) <= BF16_MEDIAN, f"{what}: the median row is off by {float(per_row.median()):.3e} (bfloat16)"
+    margin = _margins.get(id(want))
+    if margin is not None:
+        per_row = per_row[torch.cummin(margin, dim=0).values >= 0.15]
+        if per_row.numel() == 0:
+            return
+    worst_bf16_row[0] = max(worst_bf16_row[0], float(per_row.max()))
+    over = int((per_row > BF16_ROW).sum())
+    assert over <= max(1, per_row.numel() // 10), f"{what}: {over} of {per_row.numel()} rows are off by more than {BF16_ROW} (bfloat16)"
+    assert float(per_row.max()) <= BF16_WORST, f"{what}: row {int(per_row.argmax())} is off by {float(per_row.max()):.3e} (bfloat16)"
+
+
+def test_zz_report_worst_bfloat16_row():
+    print(f"worst bfloat16 row of the Fusavik comparisons: {worst_bf16_row[0]:.2e}")
+
+
+# ------------------------------------------------------------------ every mechanism alone
+
+ALONE = ["window_only", "window_plain", "decay_only", "scan_only", "scan_no_conv", "moe_only", "moe_plain", "bigram"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ALONE)
+def test_one_mechanism_whole_prompt_and_token_by_token(name, dtype):
+    """A model of one layer with one mechanism that weighs: a whole prompt, then the same tokens as a short portion
+    followed by single tokens, both equal to the plain implementation row by row."""
+    folder = folder_of(name)
+    toks = random_tokens(Z.ALL[name]["vocab"], 75, 5)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype)
+    got = replay(runner, {"w": toks}, [{"w": len(toks)}])["w"]
+    assert_close(got, want, dtype, f"{name} whole")
+    got = replay(runner, {"d": toks}, [{"d": 3}] + [{"d": 1}] * (len(toks) - 3))["d"]
+    assert_close(got, want, dtype, f"{name} token by token")
+    assert not runner.cache.live_requests()
+
+
+@pytest.mark.parametrize("name", ["window_only", "decay_only", "scan_only", "moe_only", "bigram"])
+def test_the_mechanism_matters_in_these_models(name):
+    """The comparisons above would pass with a mechanism that does nothing if it weighed nothing: with its tensors at
+    zero the plain logits move by hundreds of times the float32 tolerance."""
+    cfg, w = _model(folder_of(name))
+    toks = list(random_tokens(cfg["vocab"], 40, 5))
+    want = P.forward(toks, cfg, w)
+    dead = dict(w)
+    for key in {"window_only": ["l0.mix.left.o"], "decay_only": ["l0.mix.right.o"], "scan_only": ["l0.mix.o"], "bigram": ["bigram"],
+                "moe_only": [k for k in w if k.startswith("l0.mlp.e") and k.endswith(".down")]}[name]:
+        dead[key] = np.zeros_like(w[key])
+    assert float(np.abs(P.forward(toks, cfg, dead) - want).max() / np.abs(want).max()) > 5e-3
+    if name == "moe_only":      # the shared expert and the groups weigh as well
+        dead = dict(w)
+        dead["l0.mlp.shared.down"] = np.zeros_like(w["l0.mlp.shared.down"])
+        assert float(np.abs(P.forward(toks, cfg, dead) - want).max() / np.abs(want).max()) > 5e-3
+        free = json.loads(json.dumps(cfg))
+        del free["layers"][0]["mlp"]["router"]["groups"]
+        assert float(np.abs(P.forward(toks, free, w) - want).max() / np.abs(want).max()) > 5e-3
+
+
+# ------------------------------------------------------------------ the whole design, every schedule
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["mixed", "loop_all"])
+def test_portions_of_several_sizes_down_to_two_tokens(name, dtype):
+    folder = folder_of(name)
+    toks = random_tokens(Z.ALL[name]["vocab"], 150, 21)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype)
+    for sizes in ([150], [2], [37, 2, 23, 3], [64, 1, 1, 17], [5, 8, 16, 1]):
+        got = replay(runner, {"p": toks}, [{"p": c} for c in cuts(len(toks), sizes)])["p"]
+        assert_close(got, want, dtype, f"{name} in portions of {sizes}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("graphs", [True, False])
+def test_unequal_requests_in_one_batch_equal_each_alone_and_slots_are_used_again(dtype, graphs):
+    """Six requests of 1 to 130 tokens through a pool that holds three at a time and too few pages for all: portions
+    beside single tokens, requests that pause for a step, pages and state slots that the next request takes over as
+    they are.  Every row equals the plain implementation of its request alone."""
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    lengths = {"a": 130, "b": 1, "c": 47, "d": 80, "e": 2, "f": 66}
+    requests = {r: random_tokens(vocab, n, 40 + i) for i, (r, n) in enumerate(lengths.items())}
+    runner = runner_for(folder, dtype, max_tokens=8 * 36, max_requests=3, use_graphs=graphs)
+    steps = [{"a": 30}, {"a": 29, "b": 1, "c": 2}, {"a": 1, "c": 16}, {"c": 1, "a": 7}, {"a": 1, "c": 1}, {"a": 1, "c": 27},
+             {"a": 61}]
+    steps += [{"d": 40, "e": 1}, {"e": 1, "d": 1}, {"d": 39}]
+    steps += [{"f": 64}, {"f": 1}, {"f": 1}]
+    got = replay(runner, requests, steps)
+    for r, toks in requests.items():
+        assert_close(got[r], plain(folder, toks), dtype, f"request {r}")
+    runner.cache.check()
+    assert not runner.cache.live_requests() and runner.cache.free_pages() == runner.cache.num_pages
+    assert runner.cache.slots.num_free == 3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_in_a_batch_of_recorded_steps(dtype):
+    """Three requests decode 140 tokens each side by side after prompts of unequal length, across many page edges,
+    past the window and two edges of the attention's tiles of 64 keys, in recorded steps."""
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    prompts = {"x": 5, "y": 61, "z": 30}
+    requests = {r: random_tokens(vocab, n + 140, 70 + i) for i, (r, n) in enumerate(prompts.items())}
+    runner = runner_for(folder, dtype)
+    got = replay(runner, requests, [dict(prompts)] + [{r: 1 for r in prompts}] * 140)
+    assert any(key[0] == "d" for key in runner._recorded), "the decode steps were not recorded"
+    for r, toks in requests.items():
+        assert_close(got[r], plain(folder, toks), dtype, f"request {r}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_first_tokens_of_a_sequence(dtype):
+    """Requests of one and of two tokens, and the first rows of a longer one, on slots that a longer request has just
+    left: nothing of the request before shows (its memory, its convolution's inputs, its last token)."""
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    runner = runner_for(folder, dtype, max_requests=1)
+    long = random_tokens(vocab, 90, 3)
+    replay(runner, {"long": long}, [{"long": 90}])
+    for n in (1, 2, 5):
+        toks = random_tokens(vocab, n, 100 + n)
+        got = replay(runner, {"s": toks}, [{"s": 1}] * n)["s"]
+        assert_close(got, plain(folder, toks), dtype, f"{n} first tokens")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layer_by_layer_against_the_plain_stream(dtype):
+    """The residual stream after every run of a layer (a repeated layer counts each time), through ``Model.tap``."""
+    folder = folder_of("mixed")
+    cfg, w = _model(folder)
+    toks = list(random_tokens(cfg["vocab"], 40, 8))
+    want = []
+    P.forward(toks, cfg, w, taps=want)
+    runner = runner_for(folder, dtype, use_graphs=False)
+    got = []
+    runner.model.tap = lambda i, h: got.append(h.detach().double().cpu())
+    replay(runner, {"t": tuple(toks)}, [{"t": len(toks)}])
+    assert len(got) == len(want) == 6
+    tol = 2e-5 if dtype == "float32" else 6e-2
+    for i, (a, b) in enumerate(zip(got, want)):
+        err = float((a - torch.from_numpy(b)).abs().max() / np.abs(b).max())
+        assert err <= tol, f"layer run {i}: {err:.3e}"
+
+
+# ------------------------------------------------------------------ the window's edges and far keys, made to show
+
+def _one_hot_case(T, H, G, dk, dv, seed):
+    """Queries, keys and values such that, for a query at position i, the score of the key at position j is large
+    and positive exactly where the test says so: key j is ``e[j mod dk] * 6`` and a query is built per case."""
+    g = torch.Generator().manual_seed(seed)
+    k = torch.randn(T, G, dk, generator=g) * 0.1
+    v = torch.randn(T, G, dv, generator=g)
+    q = torch.randn(T, H, dk, generator=g) * 0.1
+    return q, k, v
+
+
+def _plain_window_softmax(q, k, v, scale, window, keep, H, G):
+    T = q.shape[0]
+    out = torch.zeros(T, H, v.shape[2], dtype=torch.float64)
+    q, k, v = q.double(), k.double(), v.double()
+    for h in range(H):
+        g = h // (H // G)
+        for i in range(T):
+            js = [j for j in range(i + 1) if P.visible(i, j, window if window is not None else T + 1, keep)]
+            s = (k[js, g] @ q[i, h]) * scale
+            p = torch.softmax(s, dim=0)
+            out[i, h] = p @ v[js, g]
+    return out.reshape(T, -1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,dk,dv,page,window,keep", [(6, 2, 16, 16, 8, 72, 6), (4, 4, 32, 48, 16, 5, 70), (3, 1, 24, 20, 4, 130, 0),
+                                                         (2, 1, 64, 64, 16, 64, 64), (5, 5, 16, 32, 8, 1, 1), (2, 2, 16, 16, 8, None, 0)])
+def test_window_edges_kept_first_tokens_and_far_keys_in_both_attention_kernels(H, G, dk, dv, page, window, keep, dtype):
+    """The attention alone over scattered pages, with one key a query made to stand out: the key just inside the
+    window, the key just outside it, the last kept first token, the first token that is not kept, and a key far back.
+    A key that is wrongly seen or wrongly missed takes or loses nearly all the weight.  Prompt portions (the
+    matrix-core kernel where it takes the sizes, else the vector units) and single tokens with the keys cut into runs
+    must both give the written-out softmax."""
+    from nanoinfer_amd import kernels as K
+    from nanoinfer_amd.kernels import stream
+    dev = torch.device("cuda")
+    T = 300
+    q, k, v = _one_hot_case(T, H, G, dk, dv, 3)
+    win = window if window is not None else T + 1
+    # per query a target key that gets a large score: cycle through the interesting places
+    for i in range(T):
+        places = [i - win + 1, i - win, keep - 1, keep, 0, i // 2, i - 63, i - 64, i - 65]
+        j = places[i % len(places)]
+        if 0 <= j <= i:
+            k[j] = k[j] + 0.0      # keys stay random; the query points at key j
+            q[i] = k[j, torch.arange(H) // (H // G)] * (160.0 / max(float(k[j].pow(2).sum(-1).max()), 1e-3))
+    scale = 0.5
+    qd, kd, vd = (t.to(dtype) for t in (q, k, v))
+    want = _plain_window_softmax(qd.float(), kd.float(), vd.float(), scale, window, keep, H, G)
+    # the cache: pages in a scattered order
+    n_pages = (T + page - 1) // page
+    perm = torch.randperm(n_pages + 5, generator=torch.Generator().manual_seed(1))[:n_pages]
+    kpool = torch.full((n_pages + 5, G, page, dk), float("nan"), dtype=dtype)
+    vpool = torch.full((n_pages + 5, G, page, dv), float("nan"), dtype=dtype)
+    for t in range(T):
+        kpool[perm[t // page], :, t % page] = kd[t]
+        vpool[perm[t // page], :, t % page] = vd[t]
+    kpool, vpool = kpool.to(dev), vpool.to(dev)
+    table = perm.to(torch.int32).view(1, -1).to(dev)
+    qrows = qd.reshape(T, H * dk).contiguous().to(dev)
+    positions = torch.arange(T, dtype=torch.int32, device=dev)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    group = H // G
+
+    def check(out, rows, what):
+        err = float((out.double().cpu() - want[rows]).abs().max() / want.abs().max())
+        assert err <= tol, f"{what}: {err:.3e}"
+
+    # a prompt of all tokens at once, and in portions that start inside the window
+    for first in (0, 100, 203):
+        n = T - first
+        for wide in (True, False):
+            rows_per = stream.bias_attention_mfma_rows(dk, dv) if wide else stream.bias_attention_rows()
+            if not rows_per:
+                continue
+            heads = min(group, rows_per)
+            tile_tokens = max(1, rows_per // heads)
+            tiles = torch.tensor(K.build_q_tiles([0], [n], [T], tile_tokens), dtype=torch.int32).view(-1, 4).to(dev)
+            out = torch.empty(n, H * dv, dtype=dtype, device=dev)
+            fn = stream.bias_attention_mfma if wide else stream.bias_attention
+            fn(qrows[first:].contiguous(), kpool, vpool, table, tiles, positions[first:].contiguous(), None, out, H, scale, 0.0, 0,
+               heads, window=window, keep_first=keep)
+            check(out, slice(first, T), f"portion from {first}, {'matrix cores' if wide else 'vector units'}")
+    # single tokens, the keys whole and cut into runs
+    heads = min(group, stream.bias_attention_rows())
+    for pos in (0, 1, keep, keep + 1, win - 1, win, win + 1, 63, 64, 65, 128, 200, 299):
+        if not 0 <= pos < T:
+            continue
+        tiles = torch.tensor(K.build_q_tiles([0], [1], [pos + 1], 1), dtype=torch.int32).view(-1, 4).to(dev)
+        for runs in (1, 3, 8):
+            out = torch.empty(1, H * dv, dtype=dtype, device=dev)
+            ws = torch.empty(H * runs * (dv + 2), dtype=torch.float32, device=dev) if runs > 1 else None
+            stream.bias_attention(qrows[pos:pos + 1].contiguous(), kpool, vpool, table, tiles, positions[pos:pos + 1].contiguous(), None,
+                                  out, H, scale, 0.0, 0, heads, runs, ws, 4, window, keep, 1.0)
+            check(out, slice(pos, pos + 1), f"single token at {pos} in {runs} runs")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_sharp_window_in_a_whole_model(dtype):
+    """The windowed model with its score factor raised until single keys decide: prompts that end, portions that start
+    and single tokens that fall just before, on and just behind the window's edge, the kept first tokens and the
+    edges of pages (8) and of the kernel's tiles of 64 keys."""
+    name = "window_only"
+    cfg = json.loads(json.dumps(Z.ALL[name]))
+    cfg["layers"][0]["mixer"]["left"]["scale"] = 6.0
+    Z.ALL["window_sharp"] = cfg
+    folder = folder_of("window_sharp")
+    toks = random_tokens(cfg["vocab"], 230, 9)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype)
+    for first in (2, 3, 4, 19, 20, 21, 23, 63, 64, 65, 127, 129):
+        rest = len(toks) - first
+        steps = [{"k": first}] + [{"k": 1}] * 3 + [{"k": c} for c in cuts(rest - 3, [62, 2, 1, 64, 3])]
+        got = replay(runner, {"k": toks}, steps)["k"]
+        assert_close(got, want, dtype, f"first portion of {first}")
+    # the rows do depend on the edge: a window one token longer or one kept token fewer moves them
+    base, w = _model(folder)
+    for key, delta in (("size", 1), ("keep_first", -1)):
+        other = json.loads(json.dumps(base))
+        other["layers"][0]["mixer"]["left"]["mask"][key] += delta
+        moved = np.abs(P.forward(list(toks[:120]), other, w) - want[:120].numpy()).max() / np.abs(want.numpy()).max()
+        assert moved > 1e-2, (key, moved)
+
+
+# ------------------------------------------------------------------ the state mixers' kernels alone
+
+@pytest.mark.parametrize("H,dk,dv", [(2, 32, 64), (3, 24, 40), (1, 8, 8), (2, 128, 16), (4, 20, 33)])
+def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv):
+    """Three sequences of unequal length in one call, continued in a second call from the state the first left, with
+    decays from strong to nearly none; against the recurrence written out in float64."""
+    from nanoinfer_amd import kernels as K
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(2)
+    lens = [37, 1, 90]
+    decay = torch.tensor([0.999, 0.3, 0.9, 0.6][:H] if H <= 4 else [0.9] * H, dtype=torch.float32)
+    width = 2 * H * dk + H * dv
+    floats = K.decay_state_floats(H, dk, dv)
+    state = torch.zeros(5, floats, device=dev)
+    state[0] = float("nan")                       # a slot that no sequence of the call owns
+    slots = torch.tensor([3, 1, 4], dtype=torch.int32, device=dev)
+    S = [torch.zeros(H, dk, dv, dtype=torch.float64) for _ in lens]
+    for _ in range(2):
+        T = sum(lens)
+        act = torch.rand(T, width, generator=g) * 0.8
+        starts = [0, lens[0], lens[0] + lens[1]]
+        out = K.decay_attention(act.to(dev), decay.to(dev), state, torch.tensor(starts, dtype=torch.int32, device=dev),
+                                torch.tensor(lens, dtype=torch.int32, device=dev), slots, H, dk, dv)
+        want = torch.zeros(T, H, dv, dtype=torch.float64)
+        a = act.double()
+        for b, (t0, n) in enumerate(zip(starts, lens)):
+            for t in range(t0, t0 + n):
+                for h in range(H):
+                    q = a[t, h * dk:(h + 1) * dk]
+                    k = a[t, H * dk + h * dk: H * dk + (h + 1) * dk]
+                    v = a[t, 2 * H * dk + h * dv: 2 * H * dk + (h + 1) * dv]
+                    S[b][h] = float(decay[h]) * S[b][h] + torch.outer(k, v)
+                    want[t, h] = S[b][h].T @ q
+        err = float((out.double().cpu() - want.reshape(T, -1)).abs().max() / want.abs().max())
+        assert err <= 5e-6, err
+    assert bool(torch.isnan(state[0]).all()) and bool(torch.isfinite(state[1:]).all())
+
+
+@pytest.mark.parametrize("inner,N,taps", [(80, 6, 4), (48, 16, 1), (33, 32, 3), (64, 3, 2), (16, 100, 2)])
+def test_convolution_and_scan_kernels_against_the_plain_recurrence(inner, N, taps):
+    """Unequal sequences, continued in a second and a third call (one of them shorter than the convolution's taps), with
+    step sizes from tiny to large; against the recurrence in float64."""
+    from nanoinfer_amd import kernels as K
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(5)
+    scan_floats = K.scan_state_floats(inner, N)
+    stride = (scan_floats + (taps - 1) * inner + 3) // 4 * 4
+    state = torch.zeros(4, stride, device=dev)
+    slots = torch.tensor([2, 0, 3], dtype=torch.int32, device=dev)
+    conv_w = torch.randn(inner, taps, generator=g) * 0.5
+    conv_b = torch.randn(inner, generator=g) * 0.1
+    A_log = torch.randn(inner, N, generator=g) * 0.7
+    A = torch.zeros(inner, scan_floats // inner)
+    A[:, :N] = -torch.exp(A_log)
+    D = torch.randn(inner, generator=g)
+    dt_b = torch.randn(inner, generator=g) * 2.0 - 1.0
+    S = [torch.zeros(inner, N, dtype=torch.float64) for _ in range(3)]
+    hist = [torch.zeros(taps - 1, inner, dtype=torch.float64) for _ in range(3)]
+    for lens in ([29, 1, 50], [1, 2, 7], [5, 1, 1]):
+        T = sum(lens)
+        starts = [0, lens[0], lens[0] + lens[1]]
+        xz = torch.randn(T, 2 * inner, generator=g)
+        dt_pre = torch.randn(T, inner, generator=g) * 2.0
+        bc = torch.randn(T, 2 * N, generator=g)
+        seq_of = torch.cat([torch.full((n,), b, dtype=torch.int32) for b, n in enumerate(lens)])
+        qs, ql = (torch.tensor(x, dtype=torch.int32, device=dev) for x in (starts, lens))
+        u32, u = K.conv_silu(xz.to(dev), inner, conv_w.to(dev), conv_b.to(dev), state, scan_floats, seq_of.to(dev), qs, ql, slots,
+                             torch.float32)
+        y = K.selective_scan(dt_pre.to(dev), dt_b.to(dev), u32, xz.to(dev), inner, bc.to(dev), A.to(dev), D.to(dev), state, qs, ql,
+                             slots, N, torch.float32)
+        want_u = torch.zeros(T, inner, dtype=torch.float64)
+        want_y = torch.zeros(T, inner, dtype=torch.float64)
+        for b, (t0, n) in enumerate(zip(starts, lens)):
+            x = torch.cat([hist[b], xz[t0:t0 + n, :inner].double()])
+            for r in range(n):
+                acc = conv_b.double().clone()
+                for j in range(taps):
+                    acc += conv_w[:, j].double() * x[r + j]
+                want_u[t0 + r] = acc / (1 + torch.exp(-acc))
+            hist[b] = x[x.shape[0] - (taps - 1):] if taps > 1 else hist[b]
+            for r in range(n):
+                t = t0 + r
+                dt = torch.nn.functional.softplus(dt_pre[t].double() + dt_b.double())
+                S[b] = torch.exp(dt[:, None] * (-torch.exp(A_log.double()))) * S[b] + (dt * want_u[t])[:, None] * bc[t, :N].double()[None, :]
+                z = xz[t, inner:].double()
+                want_y[t] = (S[b] @ bc[t, N:].double() + D.double() * want_u[t]) * (z / (1 + torch.exp(-z)))
+        assert float((u32.double().cpu() - want_u).abs().max()) <= 1e-5
+        err = float((y.double().cpu() - want_y).abs().max() / want_y.abs().max())
+        assert err <= 1e-5, err
+
+
+@pytest.mark.parametrize("E,top,groups,keep", [(8, 3, 2, 1), (6, 2, 3, 2), (5, 1, 1, 1), (12, 4, 4, 2), (4, 4, 1, 1), (70, 5, 7, 3)])
+def test_the_router_chooses_within_the_best_groups_and_weighs_by_the_softmax_over_all(E, top, groups, keep):
+    from nanoinfer_amd import kernels as K
+    g = torch.Generator().manual_seed(E)
+    z = torch.randn(40, E, generator=g) * 2.0
+    chosen, mix, mix_all = K.route_top(z.cuda(), top, mix_all=True, over_all=True, groups=groups, keep=keep)
+    router = {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}}
+    for t in range(z.shape[0]):
+        order, weight, _ = P.route(z[t].double().numpy(), router)
+        assert chosen[t].tolist() == [int(e) for e in order]
+        assert np.allclose(mix[t].cpu().numpy(), weight, rtol=2e-6, atol=1e-8)
+        dense = np.zeros(E)
+        dense[order] = weight
+        assert np.allclose(mix_all[t].cpu().numpy(), dense, rtol=2e-6, atol=1e-8)
+
+
+@pytest.mark.parametrize("ff", [24, 20])      # whole 16-byte pieces of an expert's row, and not
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_few_rows_and_many_rows_of_gated_experts_agree_with_the_plain_sum(dtype, ff):
+    from nanoinfer_amd import kernels as K
+    g = torch.Generator().manual_seed(4)
+    T, d, E, top = 12, 48, 6, 2
+    x = torch.randn(T, d, generator=g)
+    up = torch.randn(E * 2 * ff, d, generator=g) * 0.3          # an expert's gate rows, then its up rows
+    down = torch.randn(d, E * ff, generator=g) * 0.3
+    z = torch.randn(T, E, generator=g)
+    dev = torch.device("cuda")
+    xd, upd, downd = (t.to(dev, dtype).contiguous() for t in (x, up, down))
+    chosen, mix, mix_all = K.route_top(z.to(dev), top, mix_all=True, over_all=True, groups=3, keep=2)
+    x64, up64, down64 = (t.to(dtype).double() for t in (x, up, down))
+    want = torch.zeros(T, d, dtype=torch.float64)
+    for t in range(T):
+        order, weight, _ = P.route(z[t].double().numpy(), {"experts": E, "top": top, "groups": {"count": 3, "keep": 2}})
+        for e, a in zip(order, weight):
+            gate = up64[e * 2 * ff: e * 2 * ff + ff] @ x64[t]
+            lin = up64[e * 2 * ff + ff: (e + 1) * 2 * ff] @ x64[t]
+            want[t] += a * (down64[:, e * ff:(e + 1) * ff] @ (gate / (1 + torch.exp(-gate)) * lin))
+    few = K.experts_few(xd, upd, downd, chosen, mix, ff, gated=True)
+    act = K.experts_act(K.linear(xd, upd), mix_all, ff, gated=True)
+    many = K.linear(act, downd, out_dtype=torch.float32)
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    for got, what in ((few, "few rows"), (many, "many rows")):
+        err = float((got.double().cpu() - want).abs().max() / want.abs().max())
+        assert err <= tol, f"{what}: {err:.3e}"
+
+
+def test_the_stretched_rotation_is_the_plain_one():
+    """Frequencies and the factor on cos and sin as the position part gives them to the kernel."""
+    import nanoinfer_amd  # noqa: F401
+    from nanoinfer_amd.parts.standard import rope_inverse_frequencies
+    for rot in (Z.rot(16, 250000.0, (4.0, 1024, 32.0, 1.0)), Z.rot(8, 5000.0, (4.0, 64, 8.0, 1.0)), Z.rot(10, 100.0), Z.rot(64, 1e6, (40.0, 4096, 32.0, 1.0))):
+        f, amp = P.rotary_frequencies(rot)
+        sc = rot.get("scaling")
+        scaling = None if sc is None else dict(sc, kind="yarn", dims=rot["dims"], base=rot["base"])
+        got = rope_inverse_frequencies(rot["dims"], rot["base"], scaling, exact=True)
+        assert np.allclose(got, f, rtol=1e-7, atol=0)
+        if sc is not None:
+            assert abs(amp - (0.1 * np.log(sc["factor"]) + 1.0)) < 1e-12 and not np.allclose(f, P.rotary_frequencies(Z.rot(rot["dims"], rot["base"]))[0])
+
+
+# ------------------------------------------------------------------ generation through the engine's own entry point
+
+@pytest.mark.parametrize("name", ["mixed", "loop_all"])
+def test_greedy_generation_through_the_engine_is_the_plain_greedy(name):
+    """``Engine.generate`` (scheduler, chunked prompts, recorded decode runs, preemption on a pool that is too small)
+    gives the tokens that the plain implementation's argmax gives, wherever the plain logits leave no doubt."""
+    from nanoinfer_amd.engine.llm import Engine
+    from nanoinfer_amd.engine.scheduler import EngineConfig
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = folder_of(name)
+    cfg, w = _model(folder)
+    prompts = [list(random_tokens(cfg["vocab"], n, 300 + n)) for n in (3, 26, 11, 40, 1)]
+    new = 20
+    eng = Engine(folder, EngineConfig(dtype="float32", block_size=8, num_cache_blocks=10, max_sequences=3, admission_headroom=0,
+                                      prefill_chunk_size=16, max_num_batched_tokens=40), ignore_eos=True)
+    results = eng.generate(prompts, max_new_tokens=new, params=SamplingParams.greedy())
+    assert eng.scheduler.num_preemptions > 0, "the pool was meant to be too small for all"
+    checked = 0
+    for prompt, res in zip(prompts, results):
+        toks = list(prompt)
+        assert len(res.tokens) == new
+        for t in res.tokens:
+            row = P.forward(toks, cfg, w)[-1]
+            top = np.sort(row)[-2:]
+            if float(top[1] - top[0]) > 1e-3 * float(np.abs(row).max()):
+                assert t == int(row.argmax()), (len(prompt), len(toks))
+                checked += 1
+            toks.append(t)
+    assert checked >= len(prompts) * new * 3 // 4
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages() == eng.runner.cache.num_pages
+
+
+def test_sampling_with_temperature_runs_and_respects_the_seed():
+    from nanoinfer_amd.engine.llm import Engine
+    from nanoinfer_amd.engine.scheduler import EngineConfig
+    from nanoinfer_amd.sampling.params import SamplingParams
+    folder = folder_of("mixed")
+    prompts = [list(random_tokens(Z.MIXED["vocab"], n, 500 + n)) for n in (9, 20)]
+    outs = []
+    for _ in range(2):
+        eng = Engine(folder, EngineConfig(dtype="bfloat16", block_size=8, num_cache_blocks=64, max_sequences=4), ignore_eos=True)
+        outs.append([r.tokens for r in eng.generate(prompts, max_new_tokens=10,
+                                                    params=SamplingParams(temperature=0.8, top_k=20, top_p=0.9, seed=5))])
+    assert outs[0] == outs[1] and all(len(t) == 10 for t in outs[0])
+
+
+def test_the_command_line_generates_from_a_fusavik_folder(tmp_path, capsys):
+    """``bin/nanoinfer``'s program with a Fusavik ``config.json``: the random-weights mode writes the folder, the engine
+    generates greedily from two prompts, and the tokens are the plain implementation's."""
+    from nanoinfer_amd import cli
+    cfg_path, folder = str(tmp_path / "config.json"), str(tmp_path / "model")
+    with open(cfg_path, "w") as fh:
+        json.dump(Z.LOOP_ALL, fh)
+    rc = cli.main(["--random-config", cfg_path, "--save-random-model", folder, "--random-seed", "3", "--dtype", "fp32",
+                   "--prompt-ids", "5,9,77,3,120", "--prompt-len", "19", "--max-tokens", "6", "--ignore-eos", "--json",
+                   "--num-cache-blocks", "32", "--block-size", "8"])
+    assert rc == 0
+    lines = [json.loads(l) for l in capsys.readouterr().out.splitlines() if l.startswith("{")]
+    assert len(lines) == 2 and lines[0]["prompt_len"] == 5 and lines[1]["prompt_len"] == 19
+    cfg, w = P.read_model_folder(folder)
+    toks = [5, 9, 77, 3, 120]
+    for t in lines[0]["tokens"]:
+        row = P.forward(toks, cfg, w)[-1]
+        top = np.sort(row)[-2:]
+        if float(top[1] - top[0]) > 1e-3 * float(np.abs(row).max()):
+            assert t == int(row.argmax())
+        toks.append(t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_trace_program_replays_a_fusavik_model(dtype, tmp_path):
+    """``bin/trace_run`` in a process of its own, four state slots: portions beside single tokens, a request that
+    pauses, a fifth request on a slot and pages that another has given back."""
+    import subprocess
+    import sys
+    name = "mixed"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    lengths = {"a": 70, "b": 33, "c": 9, "d": 52, "e": 41}
+    requests = {r: random_tokens(vocab, n, 800 + i) for i, (r, n) in enumerate(lengths.items())}
+    plan = [{"a": 30, "b": 2}, {"a": 1, "b": 31, "c": 8, "d": 20}, {"a": 1, "c": 1, "d": 1}, {"a": 37, "d": 31},
+            {"a": 1, "e": 40}, {"e": 1}]
+    done = {r: 0 for r in requests}
+    lines, wanted = [], []
+    for i, counts in enumerate(plan):
+        entries, ended = [], []
+        for r, c in counts.items():
+            entries.append({"id": r, "tokens": list(requests[r][done[r]:done[r] + c]), "want": list(range(c))})
+            wanted.append((i, r, done[r], c))
+            done[r] += c
+            if done[r] == len(requests[r]):
+                ended.append(r)
+        lines.append(json.dumps({"step": i, "entries": entries, "end": ended}))
+    out_dir = str(tmp_path / "out")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", out_dir, "--max-tokens", "192", "--page-size", "8"],
+                          input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(plan))]
+    rows = {r: [None] * len(requests[r]) for r in requests}
+    for i in range(len(plan)):
+        data = np.fromfile(os.path.join(out_dir, f"{i}.f32"), dtype="<f4").reshape(-1, vocab)
+        at = 0
+        for step, r, first, c in wanted:
+            if step == i:
+                for j in range(c):
+                    rows[r][first + j] = torch.from_numpy(data[at + j].copy())
+                at += c
+        assert at == data.shape[0]
+    for r, toks in requests.items():
+        assert_close(torch.stack(rows[r]), plain(folder, toks), dtype, f"trace program, request {r}")
