@@ -401,20 +401,47 @@ def hybrid_config(layers: int, vocab: int, positions: int, like: dict) -> dict:
             "layers": [dict(pattern[i % 4][0], mlp=pattern[i % 4][1]) for i in range(layers)]}
 
 
+def fusavik_config(layers: int, vocab: int, like: dict) -> dict:
+    """A Fusavik model whose layers have the sizes of a Llama shape's: selective scans of twice the width with 16 numbers
+    a channel, and pairs of windowed attention (the shape's heads and head size, a window of 1,024 that keeps four first
+    tokens, half of every head rotated) beside decay attention (width / 128 heads with keys of 64 and values of 128), in
+    turn; every layer with sixteen experts of an eighth of the shape's feed-forward of which a token uses four, out of two
+    of four groups, and a shared expert of a quarter of it."""
+    width, ff, hd = like["hidden_size"], like["intermediate_size"], like["head_dim"]
+    heads = width // 128
+    pair = {"type": "parallel", "mixer": {
+        "left": {"heads": like["num_attention_heads"], "kv_heads": like["num_key_value_heads"], "dim": hd, "vdim": hd,
+                 "scale": hd ** -0.5, "mask": {"size": 1024, "keep_first": 4},
+                 "rot": {"dims": hd // 2, "base": 500000.0, "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}},
+        "right": {"heads": heads, "dim": 64, "vdim": 128, "decay": [1.0 - 2.0 ** -(2 + 6 * i / max(heads - 1, 1)) for i in range(heads)]},
+        "left_scale": 0.7, "right_scale": 0.7}}
+    scan = {"type": "mamba1", "mixer": {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4}}
+    routed = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 16, "top": 4, "groups": {"count": 4, "keep": 2}},
+              "shared": {"ff": ff // 4}}
+    pattern = [scan, pair]
+    return {"architecture": "Fusavik", "vocab": vocab, "width": width,
+            "embedding": {"scale": float(width) ** 0.5, "bigram": {"buckets": 16381, "mul_prev": 8191, "mul_cur": 31}},
+            "norm": {"eps": 1e-5}, "layers": [dict(pattern[i % 2], mlp=routed) for i in range(layers)]}
+
+
 def hybrid(args) -> int:
     """``--workload hybrid``: prefill of one prompt and decode steps of the Zekalorn shape above and of the Llama
-    shape of equal depth, one JSON line with both."""
+    shape of equal depth, one JSON line with both.  ``--workload stateful``: the same of the Fusavik shape above
+    beside the Zekalorn shape (the framework's other model with mixers that keep a state and routed experts)."""
     import torch
     torch.cuda.set_device(0)
     layers = args.layers or 8
     prompt, batch = args.prompt_len, args.batch
-    out = {"metric": "hybrid_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+    first = "fusavik" if args.workload == "stateful" else "zekalorn"
+    out = {"metric": f"{args.workload}_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
            "config": {"layers": layers, "prompt_len": prompt, "global_batch": batch, "shape": args.shape,
                       "width": SHAPES[args.shape][2]["hidden_size"], "vocab": 128256}}
     like = SHAPES[args.shape][2]
     shapes = {"zekalorn": hybrid_config(layers, 128256, prompt + 2048, like),
               "llama": dict(like, num_hidden_layers=layers, max_position_embeddings=prompt + 2048)}
+    if args.workload == "stateful":
+        shapes = {"fusavik": fusavik_config(layers, 128256, like), "zekalorn": shapes["zekalorn"]}
     for name, cfg in shapes.items():
         if args.only and name != args.only:
             continue
@@ -433,9 +460,9 @@ def hybrid(args) -> int:
         out[name] = rec
         log(f"{name}: {rec}")
         rig.close()
-    if "zekalorn" in out and f"decode_b{batch}_tok_s" in out["zekalorn"]:
-        out["value"] = out["zekalorn"][f"decode_b{batch}_tok_s"]
-        out["ms_per_step"] = out["zekalorn"][f"decode_b{batch}_step_ms"]
+    if first in out and f"decode_b{batch}_tok_s" in out[first]:
+        out["value"] = out[first][f"decode_b{batch}_tok_s"]
+        out["ms_per_step"] = out[first][f"decode_b{batch}_step_ms"]
     print(json.dumps(out))
     return 0
 
@@ -471,11 +498,12 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the further points")
     ap.add_argument("--no-further", action="store_true",
                     help="skip the points beyond the default line's: contexts of 8k and 32k, float32, the 3B shape")
-    ap.add_argument("--only", default=None, choices=["zekalorn", "llama"], help="hybrid: measure one of the two models")
-    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid"],
+    ap.add_argument("--only", default=None, choices=["zekalorn", "llama", "fusavik"], help="hybrid, stateful: measure one of the two models")
+    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid", "stateful"],
                     help="steps: the decode step and prefill of the result line's contract (default); "
                          "serving: concurrent requests through the engine's scheduler, a line of its own; "
-                         "hybrid: prefill and decode of a Zekalorn model at the 1B shape's layer sizes beside the Llama shape")
+                         "hybrid: prefill and decode of a Zekalorn model at the 1B shape's layer sizes beside the Llama shape; "
+                         "stateful: the same of a Fusavik model beside the Zekalorn one")
     ap.add_argument("--requests", type=int, default=64, help="serving: concurrent requests")
     ap.add_argument("--new-tokens", type=int, default=256, help="serving: tokens generated per request")
     ap.add_argument("--min-prompt", type=int, default=128, help="serving: shortest prompt")
@@ -496,7 +524,7 @@ def main() -> int:
         return 2
     if args.workload == "serving":
         return serving(args)
-    if args.workload == "hybrid":
+    if args.workload in ("hybrid", "stateful"):
         return hybrid(args)
     args.prefill_chunk = args.prefill_chunk or PREFILL_CHUNK
 

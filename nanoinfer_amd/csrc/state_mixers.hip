@@ -71,21 +71,38 @@ __device__ __forceinline__ void decay_load(DecayOperands& o, const float* __rest
     o.v = row[v_off];
 }
 
+// Long portions go in runs of RUN tokens, all runs at once, in three launches:
+//   1. every run on its own from an empty memory (LOCAL): its tokens' read-outs of the run's own keys, and what the run
+//      adds to the memory, L_r = sum_s decay^(last - s) k_s v_s^T, into `runs` [run][H][dv][dkp];
+//   2. decay_chain_kernel walks the runs of a sequence in order, element by element: the memory at the start of run r
+//      takes L_r's place, S <- decay^len S + L_r goes on, and the state slot gets the end;
+//   3. decay_carry_kernel adds what the memory at a run's start gives its tokens: o_t += decay^(i + 1) S_start^T q_t.
+// Run r of sequence b lies at index q_start[b] / RUN + b + r: at most T / RUN + B runs in a step.
+#define RUN 64
+
+template <bool LOCAL>
 __global__ void __launch_bounds__(256)
 decay_attention_kernel(const float* __restrict__ act, int act_stride, const float* __restrict__ decay, float* __restrict__ state,
                        size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
-                       const int32_t* __restrict__ state_slot, float* __restrict__ out, int H, int dk, int dv, int parts) {
+                       const int32_t* __restrict__ state_slot, float* __restrict__ out, int H, int dk, int dv, int parts,
+                       float* __restrict__ runs, int xblocks) {
     const int b = blockIdx.z, h = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int cols = WAVE / parts;
     const int part = lane % parts;
-    const int c = (blockIdx.x * (blockDim.x / WAVE) + wave) * cols + lane / parts;
-    const int n = q_len[b];
+    const int run = LOCAL ? blockIdx.x / xblocks : 0, xb = LOCAL ? blockIdx.x % xblocks : blockIdx.x;
+    const int c = (xb * (blockDim.x / WAVE) + wave) * cols + lane / parts;
+    const int first = run * RUN;                  // place in the portion of this block's first token
+    const int n = LOCAL ? min(q_len[b] - first, RUN) : q_len[b];
     if (c >= dv || n <= 0) return;               // whole groups of `parts` lanes leave together
     const int dkp = parts * DKPT, ch = part * DKPT;
-    float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride + (static_cast<size_t>(h) * dv + c) * dkp + ch;
+    float* srow = LOCAL ? runs + (static_cast<size_t>(q_start[b] / RUN + b + run) * H * dv + static_cast<size_t>(h) * dv + c) * dkp + ch
+                        : state + static_cast<size_t>(state_slot[b]) * state_stride + (static_cast<size_t>(h) * dv + c) * dkp + ch;
     float S[DKPT];
-    {
+    if (LOCAL) {
+#pragma unroll
+        for (int i = 0; i < DKPT; ++i) S[i] = 0.f;
+    } else {
         const float4 a = *reinterpret_cast<const float4*>(srow), d = *reinterpret_cast<const float4*>(srow + 4);
         S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
     }
@@ -93,7 +110,7 @@ decay_attention_kernel(const float* __restrict__ act, int act_stride, const floa
     const int q_off = h * dk, k_off = H * dk + h * dk, v_off = 2 * H * dk + h * dv + c;
     const bool whole = dk % DKPT == 0 && ch + DKPT <= dk && act_stride % 4 == 0;
     const bool idle = ch >= dk;                   // a lane that holds padding only
-    const int t0 = q_start[b];
+    const int t0 = q_start[b] + first;
     DecayOperands cur, nxt;
     if (!idle) decay_load(cur, act + static_cast<size_t>(t0) * act_stride, q_off, k_off, v_off, ch, dk, whole);
     for (int r = 0; r < n; ++r) {
@@ -110,9 +127,75 @@ decay_attention_kernel(const float* __restrict__ act, int act_stride, const floa
         if (part == 0) out[static_cast<size_t>(t0 + r) * (H * dv) + h * dv + c] = sum;
         cur = nxt;
     }
-    if (!idle) {
-        *reinterpret_cast<float4*>(srow) = make_float4(S[0], S[1], S[2], S[3]);
-        *reinterpret_cast<float4*>(srow + 4) = make_float4(S[4], S[5], S[6], S[7]);
+    // (a lane of padding writes back the zeros it holds: the chain over the runs reads every element)
+    *reinterpret_cast<float4*>(srow) = make_float4(S[0], S[1], S[2], S[3]);
+    *reinterpret_cast<float4*>(srow + 4) = make_float4(S[4], S[5], S[6], S[7]);
+}
+
+// step 2 of the runs: one thread an element of the memory [H][dv][dkp]
+__global__ void decay_chain_kernel(float* __restrict__ runs, const float* __restrict__ decay, float* __restrict__ state,
+                                   size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+                                   const int32_t* __restrict__ state_slot, int per_head, int elems) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    const int n = q_len[b];
+    if (e >= elems || n <= 0) return;
+    const float w = decay[e / per_head];
+    const float w_run = powf(w, static_cast<float>(RUN));
+    float* at = runs + static_cast<size_t>(q_start[b] / RUN + b) * elems + e;
+    float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride + e;
+    float S = *srow;
+    const int n_runs = (n + RUN - 1) / RUN;
+    for (int r = 0; r < n_runs; ++r) {
+        const float add = at[static_cast<size_t>(r) * elems];
+        at[static_cast<size_t>(r) * elems] = S;
+        const int len = min(RUN, n - r * RUN);
+        S = (len == RUN ? w_run : powf(w, static_cast<float>(len))) * S + add;
+    }
+    *srow = S;
+}
+
+// step 3 of the runs: the same threads as step 1, each with its eight numbers of the memory at the run's start
+__global__ void __launch_bounds__(256)
+decay_carry_kernel(const float* __restrict__ act, int act_stride, const float* __restrict__ decay, const float* __restrict__ runs,
+                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int H, int dk,
+                   int dv, int parts, int xblocks) {
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int cols = WAVE / parts;
+    const int part = lane % parts;
+    const int run = blockIdx.x / xblocks, xb = blockIdx.x % xblocks;
+    const int c = (xb * (blockDim.x / WAVE) + wave) * cols + lane / parts;
+    const int first = run * RUN;
+    const int n = min(q_len[b] - first, RUN);
+    if (c >= dv || n <= 0) return;
+    const int dkp = parts * DKPT, ch = part * DKPT;
+    const float* srow = runs + (static_cast<size_t>(q_start[b] / RUN + b + run) * H * dv + static_cast<size_t>(h) * dv + c) * dkp + ch;
+    float S[DKPT];
+    {
+        const float4 a = *reinterpret_cast<const float4*>(srow), d = *reinterpret_cast<const float4*>(srow + 4);
+        S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
+    }
+    const float w = decay[h];
+    const int q_off = h * dk + ch;
+    const bool whole = dk % DKPT == 0 && ch + DKPT <= dk && act_stride % 4 == 0;
+    const bool idle = ch >= dk;
+    const int t0 = q_start[b] + first;
+    float faded = 1.f;
+    for (int r = 0; r < n; ++r) {
+        const float* row = act + static_cast<size_t>(t0 + r) * act_stride + q_off;
+        float sum = 0.f;
+        if (!idle) {
+            if (whole) {
+                const float4 a = *reinterpret_cast<const float4*>(row), d = *reinterpret_cast<const float4*>(row + 4);
+                sum = S[0] * a.x + S[1] * a.y + S[2] * a.z + S[3] * a.w + S[4] * d.x + S[5] * d.y + S[6] * d.z + S[7] * d.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < DKPT; ++i) sum += ch + i < dk ? S[i] * row[i] : 0.f;
+            }
+        }
+        sum = parts_sum(sum, parts);
+        faded *= w;
+        if (part == 0) out[static_cast<size_t>(t0 + r) * (H * dv) + h * dv + c] += faded * sum;
     }
 }
 
@@ -122,18 +205,38 @@ NI_EXPORT int ni_decay_attention_parts(int dk) {
     return parts <= WAVE ? parts : 0;
 }
 
+NI_EXPORT int ni_state_run_tokens() { return RUN; }
+
+// `max_q_len` bounds the portions of the step; `runs` (float32, (T / RUN + B) * H * dv * dkp, or null) switches the
+// runs on: without it every sequence is walked token by token from its state.
 NI_EXPORT int ni_decay_attention(const void* act, int act_stride, const void* decay, void* state, size_t state_stride,
                                  const void* q_start, const void* q_len, const void* state_slot, void* out, int T, int B,
-                                 int H, int dk, int dv, hipStream_t stream) {
+                                 int H, int dk, int dv, int max_q_len, void* runs, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
     const int parts = ni_decay_attention_parts(dk);
     if (!parts || act_stride < 2 * H * dk + H * dv || state_stride < static_cast<size_t>(H) * dv * parts * DKPT) return -1;
     if (reinterpret_cast<uintptr_t>(state) % 16 || state_stride % 4 || reinterpret_cast<uintptr_t>(act) % 16) return -1;
     const int cols = 4 * (WAVE / parts);
-    dim3 grid((dv + cols - 1) / cols, H, B);
-    decay_attention_kernel<<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state, state_stride,
-                                                     (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot,
-                                                     (float*)out, H, dk, dv, parts);
+    const int xblocks = (dv + cols - 1) / cols;
+    if (!runs) {
+        dim3 grid(xblocks, H, B);
+        decay_attention_kernel<false><<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state,
+            state_stride, (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, H, dk, dv, parts,
+            nullptr, xblocks);
+        return NI_LAUNCH_RESULT();
+    }
+    if (max_q_len < 1 || max_q_len > T || reinterpret_cast<uintptr_t>(runs) % 16) return -1;
+    const int n_runs = (max_q_len + RUN - 1) / RUN;
+    dim3 grid(xblocks * n_runs, H, B);
+    decay_attention_kernel<true><<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state,
+        state_stride, (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, H, dk, dv, parts,
+        (float*)runs, xblocks);
+    const int elems = H * dv * parts * DKPT;
+    dim3 chain(blocks_of(elems, 256), B);
+    decay_chain_kernel<<<chain, 256, 0, stream>>>((float*)runs, (const float*)decay, (float*)state, state_stride, (const int32_t*)q_start,
+                                                  (const int32_t*)q_len, (const int32_t*)state_slot, dv * parts * DKPT, elems);
+    decay_carry_kernel<<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (const float*)runs,
+                                                 (const int32_t*)q_start, (const int32_t*)q_len, (float*)out, H, dk, dv, parts, xblocks);
     return NI_LAUNCH_RESULT();
 }
 
@@ -265,27 +368,42 @@ __device__ __forceinline__ void scan_load(ScanOperands& o, const float* __restri
     }
 }
 
-template <typename T>
+// Long portions go in runs of RUN tokens, all runs at once, as the decay attention's do:
+//   1. every run on its own from an empty state (LOCAL): sum_n S C of its own tokens' inputs into `y_local`, the step sizes
+//      summed from the run's start into `dt_sum` (both float32 [T, inner]), the state the run ends with into `runs`;
+//   2. scan_chain_kernel walks the runs of a sequence in order: the state at the start of run r takes the run's place,
+//      S <- exp(A * dt_sum at the run's end) S + the run's own goes on, the state slot gets the end;
+//   3. scan_carry_kernel adds what the state at a run's start gives its tokens, sum_n C[t, n] exp(A[c, n] dt_sum[t, c]) S_start[c, n],
+//      then D u and the gate.
+template <typename T, bool LOCAL>
 __global__ void __launch_bounds__(256)
 selective_scan_kernel(const float* __restrict__ dt_pre, const float* __restrict__ dt_bias, const float* __restrict__ u,
                       const float* __restrict__ z, int z_stride, const float* __restrict__ bc, int bc_stride,
                       const float* __restrict__ A, const float* __restrict__ D, float* __restrict__ state, size_t state_stride,
                       const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot,
-                      T* __restrict__ y, int inner, int N, int parts) {
+                      T* __restrict__ y, int inner, int N, int parts, float* __restrict__ runs, float* __restrict__ y_local,
+                      float* __restrict__ dt_sum, int xblocks) {
     const int b = blockIdx.y;
     const int part = threadIdx.x % parts;
-    const int c = (blockIdx.x * blockDim.x + threadIdx.x) / parts;
-    const int n = q_len[b];
+    const int run = LOCAL ? blockIdx.x / xblocks : 0, xb = LOCAL ? blockIdx.x % xblocks : blockIdx.x;
+    const int c = (xb * blockDim.x + threadIdx.x) / parts;
+    const int first = run * RUN;
+    const int n = LOCAL ? min(q_len[b] - first, RUN) : q_len[b];
     if (c >= inner || n <= 0) return;            // whole groups of `parts` lanes leave together
     const int np = parts * SNPT, n0 = part * SNPT;
-    float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride + static_cast<size_t>(c) * np + n0;
-    const float4 s4 = *reinterpret_cast<const float4*>(srow);
-    float S[SNPT] = {s4.x, s4.y, s4.z, s4.w};
+    float* srow = LOCAL ? runs + (static_cast<size_t>(q_start[b] / RUN + b + run) * inner + c) * np + n0
+                        : state + static_cast<size_t>(state_slot[b]) * state_stride + static_cast<size_t>(c) * np + n0;
+    float S[SNPT] = {0.f, 0.f, 0.f, 0.f};
+    if (!LOCAL) {
+        const float4 s4 = *reinterpret_cast<const float4*>(srow);
+        S[0] = s4.x; S[1] = s4.y; S[2] = s4.z; S[3] = s4.w;
+    }
     const float4 a4 = *reinterpret_cast<const float4*>(A + static_cast<size_t>(c) * np + n0);
     const float Ac[SNPT] = {a4.x, a4.y, a4.z, a4.w};
     const float bias = dt_bias[c], Dc = D[c];
     const bool whole = N % SNPT == 0 && n0 + SNPT <= N && bc_stride % 4 == 0;
-    const size_t t0 = static_cast<size_t>(q_start[b]);
+    const size_t t0 = static_cast<size_t>(q_start[b] + first);
+    float total = 0.f;
     ScanOperands cur, nxt;
     scan_load(cur, dt_pre, u, z, z_stride, bc, bc_stride, t0, c, inner, n0, N, whole);
     for (int r = 0; r < n; ++r) {
@@ -299,10 +417,85 @@ selective_scan_kernel(const float* __restrict__ dt_pre, const float* __restrict_
             sum += S[i] * cur.C[i];
         }
         sum = parts_sum(sum, parts);
-        if (part == 0) st(y + (t0 + r) * inner + c, (sum + Dc * cur.u) * silu_f(cur.z));
+        if (LOCAL) {
+            total += dt;
+            if (part == 0) {
+                y_local[(t0 + r) * inner + c] = sum;
+                dt_sum[(t0 + r) * inner + c] = total;
+            }
+        } else if (part == 0) {
+            st(y + (t0 + r) * inner + c, (sum + Dc * cur.u) * silu_f(cur.z));
+        }
         cur = nxt;
     }
     *reinterpret_cast<float4*>(srow) = make_float4(S[0], S[1], S[2], S[3]);
+}
+
+// step 2 of the runs: one thread an element of the state [inner][np]
+__global__ void scan_chain_kernel(float* __restrict__ runs, const float* __restrict__ A, const float* __restrict__ dt_sum,
+                                  float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start,
+                                  const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, int inner, int np) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    const int n = q_len[b], elems = inner * np;
+    if (e >= elems || n <= 0) return;
+    const int c = e / np;
+    const float a = A[e];
+    float* at = runs + static_cast<size_t>(q_start[b] / RUN + b) * elems + e;
+    float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride + e;
+    float S = *srow;
+    const int n_runs = (n + RUN - 1) / RUN;
+    for (int r = 0; r < n_runs; ++r) {
+        const float add = at[static_cast<size_t>(r) * elems];
+        at[static_cast<size_t>(r) * elems] = S;
+        const int last = min(n, (r + 1) * RUN) - 1;
+        S = expf(a * dt_sum[static_cast<size_t>(q_start[b] + last) * inner + c]) * S + add;
+    }
+    *srow = S;
+}
+
+// step 3 of the runs: the same threads as step 1
+template <typename T>
+__global__ void __launch_bounds__(256)
+scan_carry_kernel(const float* __restrict__ u, const float* __restrict__ z, int z_stride, const float* __restrict__ bc, int bc_stride,
+                  const float* __restrict__ A, const float* __restrict__ D, const float* __restrict__ runs,
+                  const float* __restrict__ y_local, const float* __restrict__ dt_sum, const int32_t* __restrict__ q_start,
+                  const int32_t* __restrict__ q_len, T* __restrict__ y, int inner, int N, int parts, int xblocks) {
+    const int b = blockIdx.y;
+    const int part = threadIdx.x % parts;
+    const int run = blockIdx.x / xblocks, xb = blockIdx.x % xblocks;
+    const int c = (xb * blockDim.x + threadIdx.x) / parts;
+    const int first = run * RUN;
+    const int n = min(q_len[b] - first, RUN);
+    if (c >= inner || n <= 0) return;
+    const int np = parts * SNPT, n0 = part * SNPT;
+    const float4 s4 = *reinterpret_cast<const float4*>(runs + (static_cast<size_t>(q_start[b] / RUN + b + run) * inner + c) * np + n0);
+    const float S[SNPT] = {s4.x, s4.y, s4.z, s4.w};
+    const float4 a4 = *reinterpret_cast<const float4*>(A + static_cast<size_t>(c) * np + n0);
+    const float Ac[SNPT] = {a4.x, a4.y, a4.z, a4.w};
+    const float Dc = D[c];
+    const bool whole = N % SNPT == 0 && n0 + SNPT <= N && bc_stride % 4 == 0;
+    const size_t t0 = static_cast<size_t>(q_start[b] + first);
+    for (int r = 0; r < n; ++r) {
+        const size_t t = t0 + r;
+        const float* row = bc + t * bc_stride + N + n0;
+        float C[SNPT];
+        if (whole) {
+            const float4 c4 = *reinterpret_cast<const float4*>(row);
+            C[0] = c4.x; C[1] = c4.y; C[2] = c4.z; C[3] = c4.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < SNPT; ++i) C[i] = n0 + i < N ? row[i] : 0.f;
+        }
+        const float dts = dt_sum[t * inner + c];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < SNPT; ++i) sum += C[i] * expf(Ac[i] * dts) * S[i];
+        sum = parts_sum(sum, parts);
+        if (part == 0) {
+            const float uc = u[t * inner + c];
+            st(y + t * inner + c, (y_local[t * inner + c] + sum + Dc * uc) * silu_f(z[t * z_stride + c]));
+        }
+    }
 }
 
 NI_EXPORT int ni_selective_scan_parts(int N) {
@@ -311,23 +504,49 @@ NI_EXPORT int ni_selective_scan_parts(int N) {
     return parts <= WAVE ? parts : 0;
 }
 
+template <typename T>
+static void launch_scan(const void* dt_pre, const void* dt_bias, const void* u, const void* z, int z_stride, const void* bc, int bc_stride,
+                        const void* A, const void* D, void* state, size_t state_stride, const void* q_start, const void* q_len,
+                        const void* state_slot, void* y, int B, int inner, int N, int parts, int max_q_len, void* runs, void* y_local,
+                        void* dt_sum, hipStream_t stream) {
+    const int xblocks = blocks_of(static_cast<size_t>(inner) * parts, 256);
+    if (!runs) {
+        dim3 grid(xblocks, B);
+        selective_scan_kernel<T, false><<<grid, 256, 0, stream>>>((const float*)dt_pre, (const float*)dt_bias, (const float*)u, (const float*)z,
+            z_stride, (const float*)bc, bc_stride, (const float*)A, (const float*)D, (float*)state, state_stride, (const int32_t*)q_start,
+            (const int32_t*)q_len, (const int32_t*)state_slot, (T*)y, inner, N, parts, nullptr, nullptr, nullptr, xblocks);
+        return;
+    }
+    const int n_runs = (max_q_len + RUN - 1) / RUN;
+    dim3 grid(xblocks * n_runs, B);
+    selective_scan_kernel<T, true><<<grid, 256, 0, stream>>>((const float*)dt_pre, (const float*)dt_bias, (const float*)u, (const float*)z,
+        z_stride, (const float*)bc, bc_stride, (const float*)A, (const float*)D, (float*)state, state_stride, (const int32_t*)q_start,
+        (const int32_t*)q_len, (const int32_t*)state_slot, (T*)y, inner, N, parts, (float*)runs, (float*)y_local, (float*)dt_sum, xblocks);
+    dim3 chain(blocks_of(static_cast<size_t>(inner) * parts * SNPT, 256), B);
+    scan_chain_kernel<<<chain, 256, 0, stream>>>((float*)runs, (const float*)A, (const float*)dt_sum, (float*)state, state_stride,
+                                                 (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, inner, parts * SNPT);
+    scan_carry_kernel<T><<<grid, 256, 0, stream>>>((const float*)u, (const float*)z, z_stride, (const float*)bc, bc_stride, (const float*)A,
+        (const float*)D, (const float*)runs, (const float*)y_local, (const float*)dt_sum, (const int32_t*)q_start, (const int32_t*)q_len,
+        (T*)y, inner, N, parts, xblocks);
+}
+
+// `runs` (float32, (T / RUN + B) * inner * np, or null) switches the runs on, with `y_local` and `dt_sum` (float32 [T, inner]
+// each) and `max_q_len`, a bound on the portions of the step; without it every sequence is walked token by token from its state.
 NI_EXPORT int ni_selective_scan(const void* dt_pre, const void* dt_bias, const void* u, const void* z, int z_stride, const void* bc,
                                 int bc_stride, const void* A, const void* D, void* state, size_t state_stride, const void* q_start,
-                                const void* q_len, const void* state_slot, void* y, int T, int B, int inner, int N, int dtype,
-                                hipStream_t stream) {
+                                const void* q_len, const void* state_slot, void* y, int T, int B, int inner, int N, int max_q_len,
+                                void* runs, void* y_local, void* dt_sum, int dtype, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
     const int parts = ni_selective_scan_parts(N);
     if (!parts || z_stride < inner || bc_stride < 2 * N || state_stride < static_cast<size_t>(inner) * parts * SNPT) return -1;
     if (reinterpret_cast<uintptr_t>(state) % 16 || state_stride % 4 || reinterpret_cast<uintptr_t>(A) % 16 ||
         reinterpret_cast<uintptr_t>(bc) % 16) return -1;
-    dim3 grid(blocks_of(static_cast<size_t>(inner) * parts, 256), B);
+    if (runs && (!y_local || !dt_sum || max_q_len < 1 || max_q_len > T || reinterpret_cast<uintptr_t>(runs) % 16)) return -1;
     if (dtype == 0)
-        selective_scan_kernel<float><<<grid, 256, 0, stream>>>((const float*)dt_pre, (const float*)dt_bias, (const float*)u, (const float*)z,
-            z_stride, (const float*)bc, bc_stride, (const float*)A, (const float*)D, (float*)state, state_stride, (const int32_t*)q_start,
-            (const int32_t*)q_len, (const int32_t*)state_slot, (float*)y, inner, N, parts);
+        launch_scan<float>(dt_pre, dt_bias, u, z, z_stride, bc, bc_stride, A, D, state, state_stride, q_start, q_len, state_slot, y, B,
+                           inner, N, parts, max_q_len, runs, y_local, dt_sum, stream);
     else
-        selective_scan_kernel<bf16_t><<<grid, 256, 0, stream>>>((const float*)dt_pre, (const float*)dt_bias, (const float*)u, (const float*)z,
-            z_stride, (const float*)bc, bc_stride, (const float*)A, (const float*)D, (float*)state, state_stride, (const int32_t*)q_start,
-            (const int32_t*)q_len, (const int32_t*)state_slot, (bf16_t*)y, inner, N, parts);
+        launch_scan<bf16_t>(dt_pre, dt_bias, u, z, z_stride, bc, bc_stride, A, D, state, state_stride, q_start, q_len, state_slot, y, B,
+                            inner, N, parts, max_q_len, runs, y_local, dt_sum, stream);
     return NI_LAUNCH_RESULT();
 }

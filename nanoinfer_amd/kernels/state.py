@@ -54,6 +54,14 @@ def scan_state_floats(inner: int, n: int) -> int:
     return inner * parts * 4
 
 
+STATE_RUNS_FROM = 128     # a step whose longest portion has this many tokens goes in runs of 64 tokens, all runs at once
+
+
+def _in_runs(max_q_len: int, T: int, runs) -> bool:
+    _need(0 <= max_q_len <= T, "max_q_len is larger than the step")
+    return max_q_len >= STATE_RUNS_FROM if runs is None else bool(runs)
+
+
 def silu_rows(x: torch.Tensor, n: int) -> torch.Tensor:
     """``silu`` of the first ``n`` columns of every row of ``x`` float32 [T, >= n], as float32 [T, n]."""
     T, width = x.shape
@@ -65,10 +73,14 @@ def silu_rows(x: torch.Tensor, n: int) -> torch.Tensor:
 
 
 def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-                    state_slot: torch.Tensor, H: int, dk: int, dv: int) -> torch.Tensor:
+                    state_slot: torch.Tensor, H: int, dk: int, dv: int, max_q_len: int = 0, runs=None) -> torch.Tensor:
     """Per head ``S <- decay[h] S + k v^T; o = S^T q`` over the rows of every sequence of the step, in order.
     ``act`` float32 [T, 2 H dk + H dv]: q | k | v after their activation; ``state`` float32 [slots, >=
-    decay_state_floats(H, dk, dv)], moved on by this call.  Returns ``o`` float32 [T, H dv]."""
+    decay_state_floats(H, dk, dv)], moved on by this call.  Returns ``o`` float32 [T, H dv].
+
+    ``max_q_len`` is the longest portion of the step (a host number; 0: not known).  From ``STATE_RUNS_FROM`` tokens on
+    the portions go in runs of 64 tokens that are worked out side by side and then chained (``runs`` = True / False
+    asks for one of the two ways); otherwise token by token.  Both compute the same recurrence and differ by rounding."""
     T, width = act.shape
     _gpu(act, "act", torch.float32)
     _need(width == 2 * H * dk + H * dv, "act is not q | k | v of these sizes")
@@ -77,8 +89,14 @@ def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
     _need(stride >= decay_state_floats(H, dk, dv), "the state is too small")
     B = _per_seq(q_start, q_len, state_slot)
     out = torch.empty(T, H * dv, dtype=torch.float32, device=act.device)
-    _check(state_mixers_lib().ni_decay_attention(_ptr(act), width, _ptr(decay), _ptr(state), _size_t(stride), _ptr(q_start),
-                                                 _ptr(q_len), _ptr(state_slot), _ptr(out), T, B, H, dk, dv, _stream()),
+    lib = state_mixers_lib()
+    scratch = None
+    if _in_runs(max_q_len, T, runs):
+        max_q_len = max_q_len or T
+        scratch = torch.empty((T // int(lib.ni_state_run_tokens()) + B) * decay_state_floats(H, dk, dv), dtype=torch.float32,
+                              device=act.device)
+    _check(lib.ni_decay_attention(_ptr(act), width, _ptr(decay), _ptr(state), _size_t(stride), _ptr(q_start), _ptr(q_len),
+                                  _ptr(state_slot), _ptr(out), T, B, H, dk, dv, int(max_q_len), _ptr(scratch), _stream()),
            "decay_attention")
     return out
 
@@ -127,12 +145,13 @@ def conv_silu(xz: torch.Tensor, inner: int, weight: torch.Tensor, bias: Optional
 
 def selective_scan(dt_pre: torch.Tensor, dt_bias: torch.Tensor, u: torch.Tensor, xz: torch.Tensor, z_col: int, bc: torch.Tensor,
                    A: torch.Tensor, D: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-                   state_slot: torch.Tensor, N: int, out_dtype: torch.dtype) -> torch.Tensor:
+                   state_slot: torch.Tensor, N: int, out_dtype: torch.dtype, max_q_len: int = 0, runs=None) -> torch.Tensor:
     """``dt = softplus(dt_pre + dt_bias); S <- exp(dt A) S + dt u B; y = (S . C + D u) * silu(z)`` over the rows of
     every sequence of the step, in order.  ``dt_pre``, ``u`` float32 [T, inner]; ``z``: the columns ``z_col ..`` of
     ``xz`` float32 [T, wide]; ``bc`` float32 [T, 2 N]: B | C; ``A`` float32 [inner, n padded] as
     :func:`scan_state_floats` lays a channel out (negative, padding zero); ``state`` float32 [slots, >=
-    scan_state_floats(inner, N)], moved on.  Returns y [T, inner] in ``out_dtype``."""
+    scan_state_floats(inner, N)], moved on.  Returns y [T, inner] in ``out_dtype``.  ``max_q_len`` and ``runs`` as for
+    :func:`decay_attention`."""
     T, inner = u.shape
     _gpu(u, "u", torch.float32)
     _gpu(dt_pre, "dt_pre", torch.float32, (T, inner))
@@ -148,7 +167,14 @@ def selective_scan(dt_pre: torch.Tensor, dt_bias: torch.Tensor, u: torch.Tensor,
     B = _per_seq(q_start, q_len, state_slot)
     y = torch.empty(T, inner, dtype=out_dtype, device=u.device)
     z = ctypes.c_void_p(xz.data_ptr() + 4 * z_col)
-    _check(state_mixers_lib().ni_selective_scan(_ptr(dt_pre), _ptr(dt_bias), _ptr(u), z, xz.shape[1], _ptr(bc), 2 * N, _ptr(A),
-                                                _ptr(D), _ptr(state), _size_t(stride), _ptr(q_start), _ptr(q_len), _ptr(state_slot),
-                                                _ptr(y), T, B, inner, N, dtype_code(out_dtype), _stream()), "selective_scan")
+    lib = state_mixers_lib()
+    scratch = y_local = dt_sum = None
+    if _in_runs(max_q_len, T, runs):
+        max_q_len = max_q_len or T
+        scratch = torch.empty((T // int(lib.ni_state_run_tokens()) + B) * floats, dtype=torch.float32, device=u.device)
+        y_local = torch.empty(2, T, inner, dtype=torch.float32, device=u.device)
+        y_local, dt_sum = y_local[0], y_local[1]
+    _check(lib.ni_selective_scan(_ptr(dt_pre), _ptr(dt_bias), _ptr(u), z, xz.shape[1], _ptr(bc), 2 * N, _ptr(A), _ptr(D), _ptr(state),
+                                 _size_t(stride), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(y), T, B, inner, N, int(max_q_len),
+                                 _ptr(scratch), _ptr(y_local), _ptr(dt_sum), dtype_code(out_dtype), _stream()), "selective_scan")
     return y

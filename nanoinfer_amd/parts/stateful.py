@@ -169,7 +169,7 @@ class DecayAttention(Part):
         proj = K.linear(x, self.w_in, out_dtype=torch.float32)
         act = K.silu_rows(proj, 2 * H * dk + H * dv)
         seq = ctx.per_seq
-        o = K.decay_attention(act, self.decay, cache.state, seq.q_start, seq.q_len, seq.state_slot, H, dk, dv)
+        o = K.decay_attention(act, self.decay, cache.state, seq.q_start, seq.q_len, seq.state_slot, H, dk, dv, max_q_len=ctx.max_q_len)
         y = K.gated_rmsnorm(o, proj, 2 * H * dk + H * dv, self.norm, self.eps, self.out_scale, self.rt.dtype)
         return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)
 
@@ -275,5 +275,5 @@ class SelectiveScan(Part):
         dt_pre = K.linear(K.linear(u, self.w_r), self.w_dt, out_dtype=torch.float32)
         bc = K.linear(u, self.w_bc, out_dtype=torch.float32)
         y = K.selective_scan(dt_pre, self.dt_b, u32, xz, self.inner, bc, self.A, self.D, cache.state, seq.q_start, seq.q_len,
-                             seq.state_slot, self.N, self.rt.dtype)
+                             seq.state_slot, self.N, self.rt.dtype, max_q_len=ctx.max_q_len)
         return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)

@@ -394,14 +394,16 @@ def test_a_sharp_window_in_a_whole_model(dtype):
 
 # ------------------------------------------------------------------ the state mixers' kernels alone
 
+@pytest.mark.parametrize("runs", [False, True])
 @pytest.mark.parametrize("H,dk,dv", [(2, 32, 64), (3, 24, 40), (1, 8, 8), (2, 128, 16), (4, 20, 33)])
-def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv):
+def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv, runs):
     """Three sequences of unequal length in one call, continued in a second call from the state the first left, with
-    decays from strong to nearly none; against the recurrence written out in float64."""
+    decays from strong to nearly none; against the recurrence written out in float64.  Token by token, and in runs of 64
+    tokens that are chained afterwards (sequences of one token, of a run and a bit, of less than a run)."""
     from nanoinfer_amd import kernels as K
     dev = torch.device("cuda")
     g = torch.Generator().manual_seed(2)
-    lens = [37, 1, 90]
+    lens = [37, 1, 150] if not runs else [64, 1, 203]
     decay = torch.tensor([0.999, 0.3, 0.9, 0.6][:H] if H <= 4 else [0.9] * H, dtype=torch.float32)
     width = 2 * H * dk + H * dv
     floats = K.decay_state_floats(H, dk, dv)
@@ -414,7 +416,7 @@ def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv):
         act = torch.rand(T, width, generator=g) * 0.8
         starts = [0, lens[0], lens[0] + lens[1]]
         out = K.decay_attention(act.to(dev), decay.to(dev), state, torch.tensor(starts, dtype=torch.int32, device=dev),
-                                torch.tensor(lens, dtype=torch.int32, device=dev), slots, H, dk, dv)
+                                torch.tensor(lens, dtype=torch.int32, device=dev), slots, H, dk, dv, max_q_len=max(lens), runs=runs)
         want = torch.zeros(T, H, dv, dtype=torch.float64)
         a = act.double()
         for b, (t0, n) in enumerate(zip(starts, lens)):
@@ -430,8 +432,9 @@ def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv):
     assert bool(torch.isnan(state[0]).all()) and bool(torch.isfinite(state[1:]).all())
 
 
+@pytest.mark.parametrize("runs", [False, True])
 @pytest.mark.parametrize("inner,N,taps", [(80, 6, 4), (48, 16, 1), (33, 32, 3), (64, 3, 2), (16, 100, 2)])
-def test_convolution_and_scan_kernels_against_the_plain_recurrence(inner, N, taps):
+def test_convolution_and_scan_kernels_against_the_plain_recurrence(inner, N, taps, runs):
     """Unequal sequences, continued in a second and a third call (one of them shorter than the convolution's taps), with
     step sizes from tiny to large; against the recurrence in float64."""
     from nanoinfer_amd import kernels as K
@@ -450,7 +453,7 @@ def test_convolution_and_scan_kernels_against_the_plain_recurrence(inner, N, tap
     dt_b = torch.randn(inner, generator=g) * 2.0 - 1.0
     S = [torch.zeros(inner, N, dtype=torch.float64) for _ in range(3)]
     hist = [torch.zeros(taps - 1, inner, dtype=torch.float64) for _ in range(3)]
-    for lens in ([29, 1, 50], [1, 2, 7], [5, 1, 1]):
+    for lens in ([29, 1, 50] if not runs else [129, 1, 64], [1, 2, 7] if not runs else [1, 65, 7], [5, 1, 1]):
         T = sum(lens)
         starts = [0, lens[0], lens[0] + lens[1]]
         xz = torch.randn(T, 2 * inner, generator=g)
@@ -461,7 +464,7 @@ def test_convolution_and_scan_kernels_against_the_plain_recurrence(inner, N, tap
         u32, u = K.conv_silu(xz.to(dev), inner, conv_w.to(dev), conv_b.to(dev), state, scan_floats, seq_of.to(dev), qs, ql, slots,
                              torch.float32)
         y = K.selective_scan(dt_pre.to(dev), dt_b.to(dev), u32, xz.to(dev), inner, bc.to(dev), A.to(dev), D.to(dev), state, qs, ql,
-                             slots, N, torch.float32)
+                             slots, N, torch.float32, max_q_len=max(lens), runs=runs)
         want_u = torch.zeros(T, inner, dtype=torch.float64)
         want_y = torch.zeros(T, inner, dtype=torch.float64)
         for b, (t0, n) in enumerate(zip(starts, lens)):
