@@ -78,6 +78,8 @@ __global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k
 //   the channels from `rot` on pass as they are.
 // proj float32 [T, row_stride] holds q [H * dk] | k [G * dk] | v [G * dv]; q goes to q_out [T, H * dk] in the compute
 // type, k and v into their page slots.  One workgroup a token.
+#define ROT_PAIRS 128          // rotated pairs of a head at most: heads of up to 256 channels
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const int32_t* __restrict__ positions,
@@ -85,6 +87,7 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
                           float eps, const float* __restrict__ freq, int rot, float amplitude, T* __restrict__ q_out,
                           T* __restrict__ kpool, T* __restrict__ vpool, int H, int G, int dk, int dv, int page_size) {
     __shared__ float scratch[8];
+    __shared__ float cos_of[ROT_PAIRS], sin_of[ROT_PAIRS];     // the token's angles, worked out once for all heads
     const int t = blockIdx.x, tid = threadIdx.x;
     const float* row = proj + static_cast<size_t>(t) * row_stride;
     const int nq = H * dk, nk = G * dk;
@@ -101,6 +104,15 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
     }
     const float pos = static_cast<float>(positions[t]);
     const int half = rot / 2;
+    if (freq) {
+        for (int p = tid; p < half; p += blockDim.x) {
+            float sn, cs;
+            sincosf(pos * freq[p], &sn, &cs);
+            cos_of[p] = cs * amplitude;
+            sin_of[p] = sn * amplitude;
+        }
+        __syncthreads();
+    }
     const int slot = slot_mapping ? slot_mapping[t] : -1;
     const int page = slot >= 0 ? slot / page_size : 0, in_page = slot >= 0 ? slot % page_size : 0;
     for (int i = tid; i < nq + nk; i += blockDim.x) {
@@ -114,10 +126,8 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
         if (freq && c < rot) {
             const int jp = c < half ? j + half : j - half;
             const float other = src[jp] * r * (w ? w[jp] : 1.f);
-            float sn, cs;
-            sincosf(pos * freq[c < half ? c : c - half], &sn, &cs);
-            sn *= amplitude;
-            cs *= amplitude;
+            const int p = c < half ? c : c - half;
+            const float cs = cos_of[p], sn = sin_of[p];
             v = c < half ? v * cs - other * sn : v * cs + other * sn;
         }
         if (is_q) {
@@ -141,7 +151,7 @@ NI_EXPORT int ni_qk_norm_rope_store(const void* proj, int row_stride, const void
                                     void* q_out, void* kpool, void* vpool, int T, int H, int G, int dk, int dv, int page_size,
                                     int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (rot < 0 || rot > dk || rot % 2 || row_stride < H * dk + G * dk + G * dv) return -1;
+    if (rot < 0 || rot > dk || rot % 2 || rot > 2 * ROT_PAIRS || row_stride < H * dk + G * dk + G * dv) return -1;
     if (dtype == 0)
         qk_norm_rope_store_kernel<float><<<T, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
             (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,

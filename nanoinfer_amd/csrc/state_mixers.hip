@@ -53,8 +53,9 @@ struct DecayOperands {
     float q[DKPT], k[DKPT], v;
 };
 
+// `raw`: the row holds the projections themselves and silu is applied here (steps of few tokens, which save a launch so)
 __device__ __forceinline__ void decay_load(DecayOperands& o, const float* __restrict__ row, int q_off, int k_off, int v_off,
-                                           int ch, int dk, bool whole) {
+                                           int ch, int dk, bool whole, bool raw = false) {
     if (whole) {
         const float4 a = *reinterpret_cast<const float4*>(row + q_off + ch), b = *reinterpret_cast<const float4*>(row + q_off + ch + 4);
         const float4 c = *reinterpret_cast<const float4*>(row + k_off + ch), d = *reinterpret_cast<const float4*>(row + k_off + ch + 4);
@@ -69,6 +70,14 @@ __device__ __forceinline__ void decay_load(DecayOperands& o, const float* __rest
         }
     }
     o.v = row[v_off];
+    if (raw) {
+#pragma unroll
+        for (int i = 0; i < DKPT; ++i) {
+            o.q[i] = silu_f(o.q[i]);
+            o.k[i] = silu_f(o.k[i]);
+        }
+        o.v = silu_f(o.v);
+    }
 }
 
 // Long portions go in runs of RUN tokens, all runs at once, in three launches:
@@ -85,7 +94,7 @@ __global__ void __launch_bounds__(256)
 decay_attention_kernel(const float* __restrict__ act, int act_stride, const float* __restrict__ decay, float* __restrict__ state,
                        size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
                        const int32_t* __restrict__ state_slot, float* __restrict__ out, int H, int dk, int dv, int parts,
-                       float* __restrict__ runs, int xblocks) {
+                       float* __restrict__ runs, int xblocks, bool raw) {
     const int b = blockIdx.z, h = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int cols = WAVE / parts;
@@ -112,9 +121,9 @@ decay_attention_kernel(const float* __restrict__ act, int act_stride, const floa
     const bool idle = ch >= dk;                   // a lane that holds padding only
     const int t0 = q_start[b] + first;
     DecayOperands cur, nxt;
-    if (!idle) decay_load(cur, act + static_cast<size_t>(t0) * act_stride, q_off, k_off, v_off, ch, dk, whole);
+    if (!idle) decay_load(cur, act + static_cast<size_t>(t0) * act_stride, q_off, k_off, v_off, ch, dk, whole, raw);
     for (int r = 0; r < n; ++r) {
-        if (!idle && r + 1 < n) decay_load(nxt, act + static_cast<size_t>(t0 + r + 1) * act_stride, q_off, k_off, v_off, ch, dk, whole);
+        if (!idle && r + 1 < n) decay_load(nxt, act + static_cast<size_t>(t0 + r + 1) * act_stride, q_off, k_off, v_off, ch, dk, whole, raw);
         float sum = 0.f;
         if (!idle) {
 #pragma unroll
@@ -207,12 +216,14 @@ NI_EXPORT int ni_decay_attention_parts(int dk) {
 
 NI_EXPORT int ni_state_run_tokens() { return RUN; }
 
+// `raw` 1 (token by token only): `act` holds the projections and silu is applied as they are read.
 // `max_q_len` bounds the portions of the step; `runs` (float32, (T / RUN + B) * H * dv * dkp, or null) switches the
 // runs on: without it every sequence is walked token by token from its state.
 NI_EXPORT int ni_decay_attention(const void* act, int act_stride, const void* decay, void* state, size_t state_stride,
                                  const void* q_start, const void* q_len, const void* state_slot, void* out, int T, int B,
-                                 int H, int dk, int dv, int max_q_len, void* runs, hipStream_t stream) {
+                                 int H, int dk, int dv, int max_q_len, void* runs, int raw, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
+    if (raw && runs) return -1;                   // the runs read their operands twice: they take them with silu applied
     const int parts = ni_decay_attention_parts(dk);
     if (!parts || act_stride < 2 * H * dk + H * dv || state_stride < static_cast<size_t>(H) * dv * parts * DKPT) return -1;
     if (reinterpret_cast<uintptr_t>(state) % 16 || state_stride % 4 || reinterpret_cast<uintptr_t>(act) % 16) return -1;
@@ -222,7 +233,7 @@ NI_EXPORT int ni_decay_attention(const void* act, int act_stride, const void* de
         dim3 grid(xblocks, H, B);
         decay_attention_kernel<false><<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state,
             state_stride, (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, H, dk, dv, parts,
-            nullptr, xblocks);
+            nullptr, xblocks, raw != 0);
         return NI_LAUNCH_RESULT();
     }
     if (max_q_len < 1 || max_q_len > T || reinterpret_cast<uintptr_t>(runs) % 16) return -1;
@@ -230,7 +241,7 @@ NI_EXPORT int ni_decay_attention(const void* act, int act_stride, const void* de
     dim3 grid(xblocks * n_runs, H, B);
     decay_attention_kernel<true><<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state,
         state_stride, (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, H, dk, dv, parts,
-        (float*)runs, xblocks);
+        (float*)runs, xblocks, false);
     const int elems = H * dv * parts * DKPT;
     dim3 chain(blocks_of(elems, 256), B);
     decay_chain_kernel<<<chain, 256, 0, stream>>>((float*)runs, (const float*)decay, (float*)state, state_stride, (const int32_t*)q_start,
@@ -271,20 +282,20 @@ NI_EXPORT int ni_gated_rmsnorm(const void* o, const void* gate, int gate_stride,
 //   u[t, c] = silu(bias[c] + sum_j w[c, j] * x[t - (taps - 1 - j), c])      the last tap is the token's own input
 // x is the first `inner` columns of xz float32 [T, xz_stride].  Inputs before a portion's first row come from
 // `tail` (per slot [(taps - 1)][inner], the oldest first; zero for a new sequence), which conv_tail_kernel moves on
-// afterwards, in a launch of its own.  u goes out as float32 (for the recurrence) and, if asked for, in the compute
+// afterwards, in a launch of its own (a step of single tokens, `single`, moves it on in the first kernel).  u goes out as float32 (for the recurrence) and, if asked for, in the compute
 // type (for the product that follows).
 template <typename T>
 __global__ void conv_silu_kernel(const float* __restrict__ xz, int xz_stride, const float* __restrict__ w, const float* __restrict__ bias,
-                                 const float* __restrict__ state, size_t state_stride, size_t tail_off,
+                                 float* __restrict__ state, size_t state_stride, size_t tail_off,
                                  const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
                                  const int32_t* __restrict__ state_slot, float* __restrict__ u32, T* __restrict__ uc,
-                                 int inner, int taps, size_t total) {
+                                 int inner, int taps, size_t total, bool single) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const int t = static_cast<int>(i / inner), c = static_cast<int>(i % inner);
     const int b = seq_of_token[t];
     const int r = t - q_start[b];                 // place of the token in its portion
-    const float* tail = state + static_cast<size_t>(state_slot[b]) * state_stride + tail_off;
+    float* tail = state + static_cast<size_t>(state_slot[b]) * state_stride + tail_off;
     float acc = bias ? bias[c] : 0.f;
     for (int j = 0; j < taps; ++j) {
         const int back = taps - 1 - j;            // how many tokens before this one
@@ -295,6 +306,10 @@ __global__ void conv_silu_kernel(const float* __restrict__ xz, int xz_stride, co
     const float v = silu_f(acc);
     u32[i] = v;
     if (uc) st(uc + i, v);
+    if (single) {        // every sequence brings one token: this thread alone reads and writes its channel's column of the tail
+        for (int j = 0; j + 2 < taps; ++j) tail[static_cast<size_t>(j) * inner + c] = tail[static_cast<size_t>(j + 1) * inner + c];
+        if (taps > 1) tail[static_cast<size_t>(taps - 2) * inner + c] = xz[static_cast<size_t>(t) * xz_stride + c];
+    }
 }
 
 // the last taps - 1 inputs of every sequence of the step, oldest first; a thread moves one channel's column
@@ -315,19 +330,20 @@ __global__ void conv_tail_kernel(const float* __restrict__ xz, int xz_stride, fl
 
 NI_EXPORT int ni_conv_silu(const void* xz, int xz_stride, const void* w, const void* bias, void* state, size_t state_stride,
                            size_t tail_off, const void* seq_of_token, const void* q_start, const void* q_len, const void* state_slot,
-                           void* u32, void* uc, int T, int B, int inner, int taps, int dtype, hipStream_t stream) {
+                           void* u32, void* uc, int T, int B, int inner, int taps, int single, int dtype, hipStream_t stream) {
     const size_t total = static_cast<size_t>(T) * inner;
     if (total == 0 || B <= 0) return 0;
     if (taps < 1 || xz_stride < inner || state_stride < tail_off + static_cast<size_t>(taps - 1) * inner) return -1;
+    if (single && T != B) return -1;              // a step of single tokens has one row a sequence
     if (dtype == 0)
         conv_silu_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)xz, xz_stride, (const float*)w, (const float*)bias,
-            (const float*)state, state_stride, tail_off, (const int32_t*)seq_of_token, (const int32_t*)q_start, (const int32_t*)state_slot,
-            (float*)u32, (float*)uc, inner, taps, total);
+            (float*)state, state_stride, tail_off, (const int32_t*)seq_of_token, (const int32_t*)q_start, (const int32_t*)state_slot,
+            (float*)u32, (float*)uc, inner, taps, total, single != 0);
     else
         conv_silu_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)xz, xz_stride, (const float*)w, (const float*)bias,
-            (const float*)state, state_stride, tail_off, (const int32_t*)seq_of_token, (const int32_t*)q_start, (const int32_t*)state_slot,
-            (float*)u32, (bf16_t*)uc, inner, taps, total);
-    if (taps > 1) {
+            (float*)state, state_stride, tail_off, (const int32_t*)seq_of_token, (const int32_t*)q_start, (const int32_t*)state_slot,
+            (float*)u32, (bf16_t*)uc, inner, taps, total, single != 0);
+    if (taps > 1 && !single) {
         dim3 grid(blocks_of(inner, 256), B);
         conv_tail_kernel<<<grid, 256, 0, stream>>>((const float*)xz, xz_stride, (float*)state, state_stride, tail_off,
                                                    (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, inner, taps, B);

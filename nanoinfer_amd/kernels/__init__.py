@@ -1188,5 +1188,5 @@ from .stream import (BIAS_ATTENTION_MFMA_FROM, DELTA_RUN_FROM, EXPERTS_FEW_ROWS,
                      bias_attention, bias_attention_lib, bias_attention_mfma, bias_attention_mfma_rows, bias_attention_rows, bias_attention_runs, delta_rule, delta_rule_lib, embed_scaled, experts_act, experts_few,
                      gated_side, kv_store, route_top, stream_add, stream_lib, embed_pair_hash, add_rows_vector, qk_norm_rope_store)
 # mixers with a state of fixed size: linear attention with a decay a head, the selective scan
-from .state import (conv_silu, decay_attention, decay_state_floats, gated_rmsnorm, scan_state_floats, selective_scan,  # noqa: E402,F401
+from .state import (conv_silu, decay_attention, decay_in_runs, decay_state_floats, gated_rmsnorm, scan_state_floats, selective_scan,  # noqa: E402,F401
                     silu_rows, state_mixers_lib)

@@ -62,6 +62,12 @@ def _in_runs(max_q_len: int, T: int, runs) -> bool:
     return max_q_len >= STATE_RUNS_FROM if runs is None else bool(runs)
 
 
+def decay_in_runs(max_q_len: int, T: int) -> bool:
+    """Whether :func:`decay_attention` and :func:`selective_scan` take a step of T tokens whose longest portion has
+    ``max_q_len`` in runs."""
+    return _in_runs(max_q_len, T, None)
+
+
 def silu_rows(x: torch.Tensor, n: int) -> torch.Tensor:
     """``silu`` of the first ``n`` columns of every row of ``x`` float32 [T, >= n], as float32 [T, n]."""
     T, width = x.shape
@@ -73,17 +79,20 @@ def silu_rows(x: torch.Tensor, n: int) -> torch.Tensor:
 
 
 def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-                    state_slot: torch.Tensor, H: int, dk: int, dv: int, max_q_len: int = 0, runs=None) -> torch.Tensor:
+                    state_slot: torch.Tensor, H: int, dk: int, dv: int, max_q_len: int = 0, runs=None, raw: bool = False) -> torch.Tensor:
     """Per head ``S <- decay[h] S + k v^T; o = S^T q`` over the rows of every sequence of the step, in order.
     ``act`` float32 [T, 2 H dk + H dv]: q | k | v after their activation; ``state`` float32 [slots, >=
     decay_state_floats(H, dk, dv)], moved on by this call.  Returns ``o`` float32 [T, H dv].
 
     ``max_q_len`` is the longest portion of the step (a host number; 0: not known).  From ``STATE_RUNS_FROM`` tokens on
     the portions go in runs of 64 tokens that are worked out side by side and then chained (``runs`` = True / False
-    asks for one of the two ways); otherwise token by token.  Both compute the same recurrence and differ by rounding."""
+    asks for one of the two ways); otherwise token by token.  Both compute the same recurrence and differ by rounding.
+    ``raw`` (token by token only, see :func:`decay_in_runs`): ``act`` holds the projections themselves, possibly as the
+    first columns of wider rows, and silu is applied as they are read."""
     T, width = act.shape
     _gpu(act, "act", torch.float32)
-    _need(width == 2 * H * dk + H * dv, "act is not q | k | v of these sizes")
+    _need(width >= 2 * H * dk + H * dv if raw else width == 2 * H * dk + H * dv, "act is not q | k | v of these sizes")
+    _need(not (raw and _in_runs(max_q_len, T, runs)), "the runs take their operands with silu applied")
     _gpu(decay, "decay", torch.float32, (H,))
     stride = _state(state)
     _need(stride >= decay_state_floats(H, dk, dv), "the state is too small")
@@ -96,7 +105,7 @@ def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
         scratch = torch.empty((T // int(lib.ni_state_run_tokens()) + B) * decay_state_floats(H, dk, dv), dtype=torch.float32,
                               device=act.device)
     _check(lib.ni_decay_attention(_ptr(act), width, _ptr(decay), _ptr(state), _size_t(stride), _ptr(q_start), _ptr(q_len),
-                                  _ptr(state_slot), _ptr(out), T, B, H, dk, dv, int(max_q_len), _ptr(scratch), _stream()),
+                                  _ptr(state_slot), _ptr(out), T, B, H, dk, dv, int(max_q_len), _ptr(scratch), int(bool(raw)), _stream()),
            "decay_attention")
     return out
 
@@ -119,11 +128,12 @@ def gated_rmsnorm(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, weigh
 
 def conv_silu(xz: torch.Tensor, inner: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, tail_off: int,
               seq_of_token: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, state_slot: torch.Tensor,
-              out_dtype: torch.dtype):
+              out_dtype: torch.dtype, max_q_len: int = 0):
     """``u[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - (taps - 1 - j), c])`` over the first ``inner`` columns of
     ``xz`` float32 [T, wide], the inputs before a portion's first row taken from the state's tail (per slot, from
     float ``tail_off`` on: [(taps - 1)][inner], the oldest first), which this call moves on.  Returns ``(u as
-    float32, u in out_dtype)`` (the same tensor when ``out_dtype`` is float32)."""
+    float32, u in out_dtype)`` (the same tensor when ``out_dtype`` is float32).  ``max_q_len`` 1 (a step of single
+    tokens, one row a sequence) moves the tail on in the same kernel."""
     T, wide = xz.shape
     _gpu(xz, "xz", torch.float32)
     taps = weight.shape[1]
@@ -139,7 +149,8 @@ def conv_silu(xz: torch.Tensor, inner: int, weight: torch.Tensor, bias: Optional
     uc = None if out_dtype == torch.float32 else torch.empty(T, inner, dtype=out_dtype, device=xz.device)
     _check(state_mixers_lib().ni_conv_silu(_ptr(xz), wide, _ptr(weight), _ptr(bias), _ptr(state), _size_t(stride), _size_t(tail_off),
                                            _ptr(seq_of_token), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(u32), _ptr(uc),
-                                           T, B, inner, taps, dtype_code(out_dtype), _stream()), "conv_silu")
+                                           T, B, inner, taps, int(max_q_len == 1 and T == B), dtype_code(out_dtype), _stream()),
+           "conv_silu")
     return u32, (u32 if uc is None else uc)
 
 

@@ -167,9 +167,13 @@ class DecayAttention(Part):
             raise K.KernelError("a decay_attention mixer moves its memory on: it cannot read another entry's cache")
         H, dk, dv = self.H, self.dk, self.dv
         proj = K.linear(x, self.w_in, out_dtype=torch.float32)
-        act = K.silu_rows(proj, 2 * H * dk + H * dv)
         seq = ctx.per_seq
-        o = K.decay_attention(act, self.decay, cache.state, seq.q_start, seq.q_len, seq.state_slot, H, dk, dv, max_q_len=ctx.max_q_len)
+        # long portions go in runs, which read their operands twice and want silu applied beforehand; steps of few
+        # tokens apply it as they read the projections, a launch fewer
+        raw = not K.decay_in_runs(ctx.max_q_len, x.shape[0])
+        act = proj if raw else K.silu_rows(proj, 2 * H * dk + H * dv)
+        o = K.decay_attention(act, self.decay, cache.state, seq.q_start, seq.q_len, seq.state_slot, H, dk, dv,
+                              max_q_len=ctx.max_q_len, raw=raw)
         y = K.gated_rmsnorm(o, proj, 2 * H * dk + H * dv, self.norm, self.eps, self.out_scale, self.rt.dtype)
         return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)
 
@@ -271,7 +275,7 @@ class SelectiveScan(Part):
         seq = ctx.per_seq
         xz = K.linear(x, self.w_in, out_dtype=torch.float32)
         u32, u = K.conv_silu(xz, self.inner, self.conv, self.conv_b, cache.state, self.scan_floats, ctx.seq_of_token,
-                             seq.q_start, seq.q_len, seq.state_slot, self.rt.dtype)
+                             seq.q_start, seq.q_len, seq.state_slot, self.rt.dtype, max_q_len=ctx.max_q_len)
         dt_pre = K.linear(K.linear(u, self.w_r), self.w_dt, out_dtype=torch.float32)
         bc = K.linear(u, self.w_bc, out_dtype=torch.float32)
         y = K.selective_scan(dt_pre, self.dt_b, u32, xz, self.inner, bc, self.A, self.D, cache.state, seq.q_start, seq.q_len,
