@@ -77,7 +77,9 @@ __global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k
 //   channel c + rot/2 by the angle position * freq[c], cos and sin times `amplitude` (a null freq: no rotation);
 //   the channels from `rot` on pass as they are.
 // proj float32 [T, row_stride] holds q [H * dk] | k [G * dk] | v [G * dv]; q goes to q_out [T, H * dk] in the compute
-// type, k and v into their page slots.  One workgroup a token.
+// type, k and v into their page slots.  A token is taken by gridDim.y workgroups, each with its share of the elements
+// (and the sums of squares over the whole projections, which every one of them works out): one for steps of many
+// tokens; a step of few tokens, where one workgroup a token would walk its row alone, spreads the row.
 #define ROT_PAIRS 128          // rotated pairs of a head at most: heads of up to 256 channels
 
 template <typename T>
@@ -115,7 +117,9 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
     }
     const int slot = slot_mapping ? slot_mapping[t] : -1;
     const int page = slot >= 0 ? slot / page_size : 0, in_page = slot >= 0 ? slot % page_size : 0;
-    for (int i = tid; i < nq + nk; i += blockDim.x) {
+    const int slices = gridDim.y, slice = blockIdx.y;
+    const int per = ((nq + nk + slices - 1) / slices + 3) / 4 * 4;
+    for (int i = slice * per + tid; i < min(nq + nk, (slice + 1) * per); i += blockDim.x) {
         const bool is_q = i < nq;
         const int j = is_q ? i : i - nq;                 // index inside the projection
         const float* src = is_q ? row : row + nq;
@@ -139,7 +143,8 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
     }
     if (slot >= 0) {
         const float* vsrc = row + nq + nk;
-        for (int i = tid; i < G * dv; i += blockDim.x) {
+        const int vper = (G * dv + slices - 1) / slices;
+        for (int i = slice * vper + tid; i < min(G * dv, (slice + 1) * vper); i += blockDim.x) {
             const int g = i / dv, c = i % dv;
             st(vpool + ((static_cast<size_t>(page) * G + g) * page_size + in_page) * dv + c, vsrc[i]);
         }
@@ -152,12 +157,15 @@ NI_EXPORT int ni_qk_norm_rope_store(const void* proj, int row_stride, const void
                                     int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
     if (rot < 0 || rot > dk || rot % 2 || rot > 2 * ROT_PAIRS || row_stride < H * dk + G * dk + G * dv) return -1;
+    // few tokens: a row's elements over several workgroups, one pass of 256 threads each
+    const int slices = T >= 64 ? 1 : std::max(1, std::min(16, ((H + G) * dk + 255) / 256));
+    const dim3 grid(T, slices);
     if (dtype == 0)
-        qk_norm_rope_store_kernel<float><<<T, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
+        qk_norm_rope_store_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
             (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
             (float*)q_out, (float*)kpool, (float*)vpool, H, G, dk, dv, page_size);
     else
-        qk_norm_rope_store_kernel<bf16_t><<<T, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
+        qk_norm_rope_store_kernel<bf16_t><<<grid, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
             (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
             (bf16_t*)q_out, (bf16_t*)kpool, (bf16_t*)vpool, H, G, dk, dv, page_size);
     return NI_LAUNCH_RESULT();
