@@ -379,9 +379,45 @@ __global__ void experts_act_gated_kernel(const T* __restrict__ up, const float* 
     st(act + i, v);
 }
 
+// the same, eight neighbouring elements a thread (ff a multiple of 8: they are one expert's); the elements of an
+// expert that was not chosen are not read at all
+template <typename T>
+__global__ void experts_act_gated_vec_kernel(const T* __restrict__ up, const float* __restrict__ mix_all, T* __restrict__ act,
+                                             int E, int ff, size_t pieces) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= pieces) return;
+    const size_t i = idx * 8;
+    const size_t width = static_cast<size_t>(E) * ff;
+    const size_t t = i / width;
+    const size_t in_row = i - t * width;
+    const int e = static_cast<int>(in_row / ff), c = static_cast<int>(in_row - static_cast<size_t>(e) * ff);
+    const float w = mix_all[t * E + e];
+    float v[8];
+    if (w != 0.f) {
+        const T* src = up + (t * E + e) * 2 * static_cast<size_t>(ff) + c;
+        float g[8], u[8];
+        VecIO<T, 8>::load(src, g);
+        VecIO<T, 8>::load(src + ff, u);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = w * (g[j] / (1.0f + expf(-g[j]))) * u[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = 0.f;
+    }
+    VecIO<T, 8>::store(act + i, v);
+}
+
 NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int gated, int dtype, hipStream_t stream) {
     const size_t n = static_cast<size_t>(T) * E * ff;
     if (n == 0) return 0;
+    if (gated && ff % 8 == 0 && aligned16(up, act)) {
+        const size_t pieces = n / 8;
+        if (dtype == 0)
+            experts_act_gated_vec_kernel<float><<<blocks_of(pieces, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, pieces);
+        else
+            experts_act_gated_vec_kernel<bf16_t><<<blocks_of(pieces, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, pieces);
+        return NI_LAUNCH_RESULT();
+    }
     if (gated) {
         if (dtype == 0)
             experts_act_gated_kernel<float><<<blocks_of(n, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, n);
