@@ -216,6 +216,22 @@ def test_unequal_requests_in_one_batch_equal_each_alone_and_slots_are_used_again
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["mixed", "loop_all"])
+def test_long_portions_in_runs_beside_short_ones_and_single_tokens(name, dtype):
+    """Portions long enough for the state mixers' runs of 64 tokens (a run and a bit, three runs and a bit, exactly two
+    runs) in one step with single tokens and a portion of two, continued from states that earlier steps left."""
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    lengths = {"a": 300, "b": 150, "c": 40, "d": 128}
+    requests = {r: random_tokens(vocab, n, 900 + i) for i, (r, n) in enumerate(lengths.items())}
+    runner = runner_for(folder, dtype, max_tokens=1024)
+    steps = [{"a": 200}, {"a": 1, "b": 129, "c": 2}, {"a": 99, "b": 1, "c": 1, "d": 128}, {"b": 20, "c": 37}]
+    got = replay(runner, requests, steps)
+    for r, toks in requests.items():
+        assert_close(got[r], plain(folder, toks), dtype, f"request {r}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_in_a_batch_of_recorded_steps(dtype):
     """Three requests decode 140 tokens each side by side after prompts of unequal length, across many page edges,
     past the window and two edges of the attention's tiles of 64 keys, in recorded steps."""
