@@ -80,21 +80,21 @@ __device__ __forceinline__ void decay_load(DecayOperands& o, const float* __rest
     }
 }
 
-// Long portions go in runs of RUN tokens, all runs at once, in three launches:
+// Long portions go in runs of RUN tokens (the host's choice: shorter runs for shorter portions, so that the launches
+// still fill the chip), all runs at once, in three launches:
 //   1. every run on its own from an empty memory (LOCAL): its tokens' read-outs of the run's own keys, and what the run
 //      adds to the memory, L_r = sum_s decay^(last - s) k_s v_s^T, into `runs` [run][H][dv][dkp];
 //   2. decay_chain_kernel walks the runs of a sequence in order, element by element: the memory at the start of run r
 //      takes L_r's place, S <- decay^len S + L_r goes on, and the state slot gets the end;
 //   3. decay_carry_kernel adds what the memory at a run's start gives its tokens: o_t += decay^(i + 1) S_start^T q_t.
 // Run r of sequence b lies at index q_start[b] / RUN + b + r: at most T / RUN + B runs in a step.
-#define RUN 64
 
 template <bool LOCAL>
 __global__ void __launch_bounds__(256)
 decay_attention_kernel(const float* __restrict__ act, int act_stride, const float* __restrict__ decay, float* __restrict__ state,
                        size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
                        const int32_t* __restrict__ state_slot, float* __restrict__ out, int H, int dk, int dv, int parts,
-                       float* __restrict__ runs, int xblocks, bool raw) {
+                       float* __restrict__ runs, int xblocks, bool raw, int RUN) {
     const int b = blockIdx.z, h = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int cols = WAVE / parts;
@@ -144,7 +144,7 @@ decay_attention_kernel(const float* __restrict__ act, int act_stride, const floa
 // step 2 of the runs: one thread an element of the memory [H][dv][dkp]
 __global__ void decay_chain_kernel(float* __restrict__ runs, const float* __restrict__ decay, float* __restrict__ state,
                                    size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
-                                   const int32_t* __restrict__ state_slot, int per_head, int elems) {
+                                   const int32_t* __restrict__ state_slot, int per_head, int elems, int RUN) {
     const int e = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
     const int n = q_len[b];
     if (e >= elems || n <= 0) return;
@@ -167,7 +167,7 @@ __global__ void decay_chain_kernel(float* __restrict__ runs, const float* __rest
 __global__ void __launch_bounds__(256)
 decay_carry_kernel(const float* __restrict__ act, int act_stride, const float* __restrict__ decay, const float* __restrict__ runs,
                    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int H, int dk,
-                   int dv, int parts, int xblocks) {
+                   int dv, int parts, int xblocks, int RUN) {
     const int b = blockIdx.z, h = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int cols = WAVE / parts;
@@ -214,14 +214,12 @@ NI_EXPORT int ni_decay_attention_parts(int dk) {
     return parts <= WAVE ? parts : 0;
 }
 
-NI_EXPORT int ni_state_run_tokens() { return RUN; }
-
 // `raw` 1 (token by token only): `act` holds the projections and silu is applied as they are read.
 // `max_q_len` bounds the portions of the step; `runs` (float32, (T / RUN + B) * H * dv * dkp, or null) switches the
 // runs on: without it every sequence is walked token by token from its state.
 NI_EXPORT int ni_decay_attention(const void* act, int act_stride, const void* decay, void* state, size_t state_stride,
                                  const void* q_start, const void* q_len, const void* state_slot, void* out, int T, int B,
-                                 int H, int dk, int dv, int max_q_len, void* runs, int raw, hipStream_t stream) {
+                                 int H, int dk, int dv, int max_q_len, void* runs, int RUN, int raw, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
     if (raw && runs) return -1;                   // the runs read their operands twice: they take them with silu applied
     const int parts = ni_decay_attention_parts(dk);
@@ -233,21 +231,21 @@ NI_EXPORT int ni_decay_attention(const void* act, int act_stride, const void* de
         dim3 grid(xblocks, H, B);
         decay_attention_kernel<false><<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state,
             state_stride, (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, H, dk, dv, parts,
-            nullptr, xblocks, raw != 0);
+            nullptr, xblocks, raw != 0, 0);
         return NI_LAUNCH_RESULT();
     }
-    if (max_q_len < 1 || max_q_len > T || reinterpret_cast<uintptr_t>(runs) % 16) return -1;
+    if (max_q_len < 1 || max_q_len > T || RUN < 1 || reinterpret_cast<uintptr_t>(runs) % 16) return -1;
     const int n_runs = (max_q_len + RUN - 1) / RUN;
     dim3 grid(xblocks * n_runs, H, B);
     decay_attention_kernel<true><<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (float*)state,
         state_stride, (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, H, dk, dv, parts,
-        (float*)runs, xblocks, false);
+        (float*)runs, xblocks, false, RUN);
     const int elems = H * dv * parts * DKPT;
     dim3 chain(blocks_of(elems, 256), B);
     decay_chain_kernel<<<chain, 256, 0, stream>>>((float*)runs, (const float*)decay, (float*)state, state_stride, (const int32_t*)q_start,
-                                                  (const int32_t*)q_len, (const int32_t*)state_slot, dv * parts * DKPT, elems);
+                                                  (const int32_t*)q_len, (const int32_t*)state_slot, dv * parts * DKPT, elems, RUN);
     decay_carry_kernel<<<grid, 256, 0, stream>>>((const float*)act, act_stride, (const float*)decay, (const float*)runs,
-                                                 (const int32_t*)q_start, (const int32_t*)q_len, (float*)out, H, dk, dv, parts, xblocks);
+                                                 (const int32_t*)q_start, (const int32_t*)q_len, (float*)out, H, dk, dv, parts, xblocks, RUN);
     return NI_LAUNCH_RESULT();
 }
 
@@ -264,17 +262,22 @@ gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ gate
     for (int i = threadIdx.x; i < n; i += blockDim.x) ss += row[i] * row[i];
     const float r = out_scale / sqrtf(block_sum(ss, scratch) / static_cast<float>(n) + eps);
     const float* g = gate + static_cast<size_t>(t) * gate_stride;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) st(y + static_cast<size_t>(t) * n + i, row[i] * r * w[i] * sigmoid_f(g[i]));
+    // a token is taken by gridDim.y workgroups, each with its share of the elements (and the whole row's sum of squares)
+    const int per = (n + gridDim.y - 1) / gridDim.y;
+    for (int i = blockIdx.y * per + threadIdx.x; i < min(n, (blockIdx.y + 1) * per); i += blockDim.x)
+        st(y + static_cast<size_t>(t) * n + i, row[i] * r * w[i] * sigmoid_f(g[i]));
 }
 
 NI_EXPORT int ni_gated_rmsnorm(const void* o, const void* gate, int gate_stride, const void* w, void* y, int T, int n, float eps,
                                float out_scale, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
     if (gate_stride < n) return -1;
+    // few tokens: a row's elements over several workgroups (one workgroup walking a long row alone is a chain of round trips)
+    const dim3 grid(T, T >= 64 ? 1 : std::max(1, std::min(16, (n + 255) / 256)));
     if (dtype == 0)
-        gated_rmsnorm_kernel<float><<<T, 256, 0, stream>>>((const float*)o, (const float*)gate, gate_stride, (const float*)w, (float*)y, n, eps, out_scale);
+        gated_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>((const float*)o, (const float*)gate, gate_stride, (const float*)w, (float*)y, n, eps, out_scale);
     else
-        gated_rmsnorm_kernel<bf16_t><<<T, 256, 0, stream>>>((const float*)o, (const float*)gate, gate_stride, (const float*)w, (bf16_t*)y, n, eps, out_scale);
+        gated_rmsnorm_kernel<bf16_t><<<grid, 256, 0, stream>>>((const float*)o, (const float*)gate, gate_stride, (const float*)w, (bf16_t*)y, n, eps, out_scale);
     return NI_LAUNCH_RESULT();
 }
 
@@ -398,7 +401,7 @@ selective_scan_kernel(const float* __restrict__ dt_pre, const float* __restrict_
                       const float* __restrict__ A, const float* __restrict__ D, float* __restrict__ state, size_t state_stride,
                       const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot,
                       T* __restrict__ y, int inner, int N, int parts, float* __restrict__ runs, float* __restrict__ y_local,
-                      float* __restrict__ dt_sum, int xblocks) {
+                      float* __restrict__ dt_sum, int xblocks, int RUN) {
     const int b = blockIdx.y;
     const int part = threadIdx.x % parts;
     const int run = LOCAL ? blockIdx.x / xblocks : 0, xb = LOCAL ? blockIdx.x % xblocks : blockIdx.x;
@@ -450,7 +453,7 @@ selective_scan_kernel(const float* __restrict__ dt_pre, const float* __restrict_
 // step 2 of the runs: one thread an element of the state [inner][np]
 __global__ void scan_chain_kernel(float* __restrict__ runs, const float* __restrict__ A, const float* __restrict__ dt_sum,
                                   float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start,
-                                  const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, int inner, int np) {
+                                  const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, int inner, int np, int RUN) {
     const int e = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
     const int n = q_len[b], elems = inner * np;
     if (e >= elems || n <= 0) return;
@@ -475,7 +478,7 @@ __global__ void __launch_bounds__(256)
 scan_carry_kernel(const float* __restrict__ u, const float* __restrict__ z, int z_stride, const float* __restrict__ bc, int bc_stride,
                   const float* __restrict__ A, const float* __restrict__ D, const float* __restrict__ runs,
                   const float* __restrict__ y_local, const float* __restrict__ dt_sum, const int32_t* __restrict__ q_start,
-                  const int32_t* __restrict__ q_len, T* __restrict__ y, int inner, int N, int parts, int xblocks) {
+                  const int32_t* __restrict__ q_len, T* __restrict__ y, int inner, int N, int parts, int xblocks, int RUN) {
     const int b = blockIdx.y;
     const int part = threadIdx.x % parts;
     const int run = blockIdx.x / xblocks, xb = blockIdx.x % xblocks;
@@ -524,26 +527,26 @@ template <typename T>
 static void launch_scan(const void* dt_pre, const void* dt_bias, const void* u, const void* z, int z_stride, const void* bc, int bc_stride,
                         const void* A, const void* D, void* state, size_t state_stride, const void* q_start, const void* q_len,
                         const void* state_slot, void* y, int B, int inner, int N, int parts, int max_q_len, void* runs, void* y_local,
-                        void* dt_sum, hipStream_t stream) {
+                        void* dt_sum, int RUN, hipStream_t stream) {
     const int xblocks = blocks_of(static_cast<size_t>(inner) * parts, 256);
     if (!runs) {
         dim3 grid(xblocks, B);
         selective_scan_kernel<T, false><<<grid, 256, 0, stream>>>((const float*)dt_pre, (const float*)dt_bias, (const float*)u, (const float*)z,
             z_stride, (const float*)bc, bc_stride, (const float*)A, (const float*)D, (float*)state, state_stride, (const int32_t*)q_start,
-            (const int32_t*)q_len, (const int32_t*)state_slot, (T*)y, inner, N, parts, nullptr, nullptr, nullptr, xblocks);
+            (const int32_t*)q_len, (const int32_t*)state_slot, (T*)y, inner, N, parts, nullptr, nullptr, nullptr, xblocks, 0);
         return;
     }
     const int n_runs = (max_q_len + RUN - 1) / RUN;
     dim3 grid(xblocks * n_runs, B);
     selective_scan_kernel<T, true><<<grid, 256, 0, stream>>>((const float*)dt_pre, (const float*)dt_bias, (const float*)u, (const float*)z,
         z_stride, (const float*)bc, bc_stride, (const float*)A, (const float*)D, (float*)state, state_stride, (const int32_t*)q_start,
-        (const int32_t*)q_len, (const int32_t*)state_slot, (T*)y, inner, N, parts, (float*)runs, (float*)y_local, (float*)dt_sum, xblocks);
+        (const int32_t*)q_len, (const int32_t*)state_slot, (T*)y, inner, N, parts, (float*)runs, (float*)y_local, (float*)dt_sum, xblocks, RUN);
     dim3 chain(blocks_of(static_cast<size_t>(inner) * parts * SNPT, 256), B);
     scan_chain_kernel<<<chain, 256, 0, stream>>>((float*)runs, (const float*)A, (const float*)dt_sum, (float*)state, state_stride,
-                                                 (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, inner, parts * SNPT);
+                                                 (const int32_t*)q_start, (const int32_t*)q_len, (const int32_t*)state_slot, inner, parts * SNPT, RUN);
     scan_carry_kernel<T><<<grid, 256, 0, stream>>>((const float*)u, (const float*)z, z_stride, (const float*)bc, bc_stride, (const float*)A,
         (const float*)D, (const float*)runs, (const float*)y_local, (const float*)dt_sum, (const int32_t*)q_start, (const int32_t*)q_len,
-        (T*)y, inner, N, parts, xblocks);
+        (T*)y, inner, N, parts, xblocks, RUN);
 }
 
 // `runs` (float32, (T / RUN + B) * inner * np, or null) switches the runs on, with `y_local` and `dt_sum` (float32 [T, inner]
@@ -551,18 +554,18 @@ static void launch_scan(const void* dt_pre, const void* dt_bias, const void* u, 
 NI_EXPORT int ni_selective_scan(const void* dt_pre, const void* dt_bias, const void* u, const void* z, int z_stride, const void* bc,
                                 int bc_stride, const void* A, const void* D, void* state, size_t state_stride, const void* q_start,
                                 const void* q_len, const void* state_slot, void* y, int T, int B, int inner, int N, int max_q_len,
-                                void* runs, void* y_local, void* dt_sum, int dtype, hipStream_t stream) {
+                                void* runs, void* y_local, void* dt_sum, int RUN, int dtype, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
     const int parts = ni_selective_scan_parts(N);
     if (!parts || z_stride < inner || bc_stride < 2 * N || state_stride < static_cast<size_t>(inner) * parts * SNPT) return -1;
     if (reinterpret_cast<uintptr_t>(state) % 16 || state_stride % 4 || reinterpret_cast<uintptr_t>(A) % 16 ||
         reinterpret_cast<uintptr_t>(bc) % 16) return -1;
-    if (runs && (!y_local || !dt_sum || max_q_len < 1 || max_q_len > T || reinterpret_cast<uintptr_t>(runs) % 16)) return -1;
+    if (runs && (!y_local || !dt_sum || max_q_len < 1 || max_q_len > T || RUN < 1 || reinterpret_cast<uintptr_t>(runs) % 16)) return -1;
     if (dtype == 0)
         launch_scan<float>(dt_pre, dt_bias, u, z, z_stride, bc, bc_stride, A, D, state, state_stride, q_start, q_len, state_slot, y, B,
-                           inner, N, parts, max_q_len, runs, y_local, dt_sum, stream);
+                           inner, N, parts, max_q_len, runs, y_local, dt_sum, RUN, stream);
     else
         launch_scan<bf16_t>(dt_pre, dt_bias, u, z, z_stride, bc, bc_stride, A, D, state, state_stride, q_start, q_len, state_slot, y, B,
-                            inner, N, parts, max_q_len, runs, y_local, dt_sum, stream);
+                            inner, N, parts, max_q_len, runs, y_local, dt_sum, RUN, stream);
     return NI_LAUNCH_RESULT();
 }

@@ -229,12 +229,23 @@ NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int
 // an expert was not chosen.
 // One wavefront a row: a lane keeps the logits of experts lane, lane + 64, ...; each of the `top` rounds finds the
 // largest logit not yet taken (the lowest index among equal ones) by two butterflies over the lanes.
+template <int SLOTS>
 __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen, float* __restrict__ mix,
                                  float* __restrict__ mix_all, int T, int E, int top, int over_all, int n_groups, int keep) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* row = z + static_cast<size_t>(t) * E;
     int32_t* c = chosen + static_cast<size_t>(t) * top;
     float* m = mix + static_cast<size_t>(t) * top;
+    // the row once, into registers: slot j of a lane is expert lane + 64 j (every round below would else wait for memory
+    // again); a logit that is no number is never preferred
+    float vals[SLOTS];
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) {
+        const int e = lane + j * WAVE;
+        float ze = e < E ? row[e] : -INFINITY;
+        if (!(ze == ze)) ze = -INFINITY;
+        vals[j] = ze;
+    }
     float best = 0.f, total = 0.f;
     unsigned taken_mask = 0;        // bit j: this lane's expert lane + 64 j has been chosen
     if (mix_all) {                  // zeros first; the fence lets them land before lane 0 writes the chosen ones at the end
@@ -248,8 +259,11 @@ __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restric
         float mine = -INFINITY;
         for (int g = 0; g < n_groups; ++g) {
             float v = -INFINITY;
-            for (int e = lane; e < E; e += WAVE)
-                if (e / per_group == g) { const float ze = row[e]; if (ze == ze) v = fmaxf(v, ze); }
+#pragma unroll
+            for (int j = 0; j < SLOTS; ++j) {
+                const int e = lane + j * WAVE;
+                if (e < E && e / per_group == g) v = fmaxf(v, vals[j]);
+            }
             v = wave_max(v);
             if (lane == g) mine = v;
         }
@@ -268,21 +282,25 @@ __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restric
     }
     if (over_all) {                 // the softmax runs over every expert, chosen or not
         float v = -INFINITY;
-        for (int e = lane; e < E; e += WAVE) { const float ze = row[e]; if (ze == ze) v = fmaxf(v, ze); }
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j) v = fmaxf(v, vals[j]);
         best = wave_max(v);
         float sum = 0.f;
-        for (int e = lane; e < E; e += WAVE) { const float ze = row[e]; if (ze == ze) sum += expf(ze - best); }
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j)
+            if (lane + j * WAVE < E && vals[j] > -INFINITY) sum += expf(vals[j] - best);
         total = wave_sum(sum);
     }
     for (int k = 0; k < top; ++k) {
         float v = -INFINITY;
         int at = 0x7fffffff;
-        for (int e = lane; e < E; e += WAVE) {
-            const bool taken = (taken_mask >> (e / WAVE)) & 1u;
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j) {
+            const int e = lane + j * WAVE;
+            if (e >= E) continue;
+            const bool taken = (taken_mask >> j) & 1u;
             const bool open = (open_groups >> (n_groups > 1 ? e / per_group : 0)) & 1ull;
-            float ze = row[e];
-            if (!(ze == ze)) ze = -INFINITY;       // a logit that is no number is never preferred
-            if (!taken && open && (at == 0x7fffffff || ze > v)) { at = e; v = ze; }
+            if (!taken && open && (at == 0x7fffffff || vals[j] > v)) { at = e; v = vals[j]; }
         }
         const float vmax = wave_max(v);
         int cand = (at != 0x7fffffff && v == vmax) ? at : 0x7fffffff;
@@ -308,8 +326,15 @@ NI_EXPORT int ni_route_top(const void* z, void* chosen, void* mix, void* mix_all
     if (T <= 0) return 0;
     if (top < 1 || top > E || E > 32 * WAVE) return -1;
     if (n_groups < 1 || n_groups > WAVE || E % n_groups || keep < 1 || keep > n_groups || top > E / n_groups * keep) return -1;
-    route_top_kernel<<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
-                                             over_all, n_groups, keep);
+    if (E <= WAVE)
+        route_top_kernel<1><<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
+                                                    over_all, n_groups, keep);
+    else if (E <= 4 * WAVE)
+        route_top_kernel<4><<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
+                                                    over_all, n_groups, keep);
+    else
+        route_top_kernel<32><<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
+                                                     over_all, n_groups, keep);
     return NI_LAUNCH_RESULT();
 }
 

@@ -54,7 +54,17 @@ def scan_state_floats(inner: int, n: int) -> int:
     return inner * parts * 4
 
 
-STATE_RUNS_FROM = 128     # a step whose longest portion has this many tokens goes in runs of 64 tokens, all runs at once
+STATE_RUNS_FROM = 64      # a step whose longest portion has this many tokens goes in runs of tokens, all runs at once
+
+
+def run_tokens(T: int, columns: int) -> int:
+    """Tokens of a run for a step of T tokens whose token-by-token kernel has ``columns`` workgroups a sequence: 64, or
+    less (a power of two, at least 16) where runs of 64 would leave the launches under about 2,048 workgroups: a run is
+    a chain of dependent steps, and only many runs at once hide their round trips to memory."""
+    run = 64
+    while run > 16 and (T // run) * max(columns, 1) < 2048:
+        run //= 2
+    return run
 
 
 def _in_runs(max_q_len: int, T: int, runs) -> bool:
@@ -79,14 +89,15 @@ def silu_rows(x: torch.Tensor, n: int) -> torch.Tensor:
 
 
 def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-                    state_slot: torch.Tensor, H: int, dk: int, dv: int, max_q_len: int = 0, runs=None, raw: bool = False) -> torch.Tensor:
+                    state_slot: torch.Tensor, H: int, dk: int, dv: int, max_q_len: int = 0, runs=None, raw: bool = False,
+                    run_len: Optional[int] = None) -> torch.Tensor:
     """Per head ``S <- decay[h] S + k v^T; o = S^T q`` over the rows of every sequence of the step, in order.
     ``act`` float32 [T, 2 H dk + H dv]: q | k | v after their activation; ``state`` float32 [slots, >=
     decay_state_floats(H, dk, dv)], moved on by this call.  Returns ``o`` float32 [T, H dv].
 
     ``max_q_len`` is the longest portion of the step (a host number; 0: not known).  From ``STATE_RUNS_FROM`` tokens on
-    the portions go in runs of 64 tokens that are worked out side by side and then chained (``runs`` = True / False
-    asks for one of the two ways); otherwise token by token.  Both compute the same recurrence and differ by rounding.
+    the portions go in runs of :func:`run_tokens` tokens (``run_len``: of that many) that are worked out side by side
+    and then chained (``runs`` = True / False asks for one of the two ways); otherwise token by token.  Both compute the same recurrence and differ by rounding.
     ``raw`` (token by token only, see :func:`decay_in_runs`): ``act`` holds the projections themselves, possibly as the
     first columns of wider rows, and silu is applied as they are read."""
     T, width = act.shape
@@ -99,13 +110,14 @@ def decay_attention(act: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
     B = _per_seq(q_start, q_len, state_slot)
     out = torch.empty(T, H * dv, dtype=torch.float32, device=act.device)
     lib = state_mixers_lib()
-    scratch = None
+    scratch, run = None, 0
     if _in_runs(max_q_len, T, runs):
         max_q_len = max_q_len or T
-        scratch = torch.empty((T // int(lib.ni_state_run_tokens()) + B) * decay_state_floats(H, dk, dv), dtype=torch.float32,
-                              device=act.device)
+        parts = _pow2_parts(dk, 8)
+        run = run_tokens(T, H * -(-dv // (4 * (64 // parts)))) if run_len is None else int(run_len)
+        scratch = torch.empty((T // run + B) * decay_state_floats(H, dk, dv), dtype=torch.float32, device=act.device)
     _check(lib.ni_decay_attention(_ptr(act), width, _ptr(decay), _ptr(state), _size_t(stride), _ptr(q_start), _ptr(q_len),
-                                  _ptr(state_slot), _ptr(out), T, B, H, dk, dv, int(max_q_len), _ptr(scratch), int(bool(raw)), _stream()),
+                                  _ptr(state_slot), _ptr(out), T, B, H, dk, dv, int(max_q_len), _ptr(scratch), run, int(bool(raw)), _stream()),
            "decay_attention")
     return out
 
@@ -156,7 +168,8 @@ def conv_silu(xz: torch.Tensor, inner: int, weight: torch.Tensor, bias: Optional
 
 def selective_scan(dt_pre: torch.Tensor, dt_bias: torch.Tensor, u: torch.Tensor, xz: torch.Tensor, z_col: int, bc: torch.Tensor,
                    A: torch.Tensor, D: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-                   state_slot: torch.Tensor, N: int, out_dtype: torch.dtype, max_q_len: int = 0, runs=None) -> torch.Tensor:
+                   state_slot: torch.Tensor, N: int, out_dtype: torch.dtype, max_q_len: int = 0, runs=None,
+                   run_len: Optional[int] = None) -> torch.Tensor:
     """``dt = softplus(dt_pre + dt_bias); S <- exp(dt A) S + dt u B; y = (S . C + D u) * silu(z)`` over the rows of
     every sequence of the step, in order.  ``dt_pre``, ``u`` float32 [T, inner]; ``z``: the columns ``z_col ..`` of
     ``xz`` float32 [T, wide]; ``bc`` float32 [T, 2 N]: B | C; ``A`` float32 [inner, n padded] as
@@ -180,12 +193,14 @@ def selective_scan(dt_pre: torch.Tensor, dt_bias: torch.Tensor, u: torch.Tensor,
     z = ctypes.c_void_p(xz.data_ptr() + 4 * z_col)
     lib = state_mixers_lib()
     scratch = y_local = dt_sum = None
+    run = 0
     if _in_runs(max_q_len, T, runs):
         max_q_len = max_q_len or T
-        scratch = torch.empty((T // int(lib.ni_state_run_tokens()) + B) * floats, dtype=torch.float32, device=u.device)
+        run = run_tokens(T, -(-floats // 4 // 256)) if run_len is None else int(run_len)
+        scratch = torch.empty((T // run + B) * floats, dtype=torch.float32, device=u.device)
         y_local = torch.empty(2, T, inner, dtype=torch.float32, device=u.device)
         y_local, dt_sum = y_local[0], y_local[1]
     _check(lib.ni_selective_scan(_ptr(dt_pre), _ptr(dt_bias), _ptr(u), z, xz.shape[1], _ptr(bc), 2 * N, _ptr(A), _ptr(D), _ptr(state),
                                  _size_t(stride), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(y), T, B, inner, N, int(max_q_len),
-                                 _ptr(scratch), _ptr(y_local), _ptr(dt_sum), dtype_code(out_dtype), _stream()), "selective_scan")
+                                 _ptr(scratch), _ptr(y_local), _ptr(dt_sum), run, dtype_code(out_dtype), _stream()), "selective_scan")
     return y

@@ -414,8 +414,8 @@ def test_a_sharp_window_in_a_whole_model(dtype):
 @pytest.mark.parametrize("H,dk,dv", [(2, 32, 64), (3, 24, 40), (1, 8, 8), (2, 128, 16), (4, 20, 33)])
 def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv, runs):
     """Three sequences of unequal length in one call, continued in a second call from the state the first left, with
-    decays from strong to nearly none; against the recurrence written out in float64.  Token by token, and in runs of 64
-    tokens that are chained afterwards (sequences of one token, of a run and a bit, of less than a run)."""
+    decays from strong to nearly none; against the recurrence written out in float64.  Token by token, and in runs of 16 or
+    64 tokens that are chained afterwards (sequences of one token, of a run and a bit, of less than a run)."""
     from nanoinfer_amd import kernels as K
     dev = torch.device("cuda")
     g = torch.Generator().manual_seed(2)
@@ -432,7 +432,8 @@ def test_decay_attention_kernel_against_the_plain_recurrence(H, dk, dv, runs):
         act = torch.rand(T, width, generator=g) * 0.8
         starts = [0, lens[0], lens[0] + lens[1]]
         out = K.decay_attention(act.to(dev), decay.to(dev), state, torch.tensor(starts, dtype=torch.int32, device=dev),
-                                torch.tensor(lens, dtype=torch.int32, device=dev), slots, H, dk, dv, max_q_len=max(lens), runs=runs)
+                                torch.tensor(lens, dtype=torch.int32, device=dev), slots, H, dk, dv, max_q_len=max(lens), runs=runs,
+                                run_len=(64 if H == 2 else None) if runs else None)      # runs of 64, and of what the step's size asks for
         want = torch.zeros(T, H, dv, dtype=torch.float64)
         a = act.double()
         for b, (t0, n) in enumerate(zip(starts, lens)):
@@ -480,7 +481,7 @@ def test_convolution_and_scan_kernels_against_the_plain_recurrence(inner, N, tap
         u32, u = K.conv_silu(xz.to(dev), inner, conv_w.to(dev), conv_b.to(dev), state, scan_floats, seq_of.to(dev), qs, ql, slots,
                              torch.float32)
         y = K.selective_scan(dt_pre.to(dev), dt_b.to(dev), u32, xz.to(dev), inner, bc.to(dev), A.to(dev), D.to(dev), state, qs, ql,
-                             slots, N, torch.float32, max_q_len=max(lens), runs=runs)
+                             slots, N, torch.float32, max_q_len=max(lens), runs=runs, run_len=(64 if taps == 3 else None) if runs else None)
         want_u = torch.zeros(T, inner, dtype=torch.float64)
         want_y = torch.zeros(T, inner, dtype=torch.float64)
         for b, (t0, n) in enumerate(zip(starts, lens)):
