@@ -273,7 +273,11 @@ def bias_attention_runs(n_tiles: int, kv_heads: int, head_chunks: int, max_keys:
     blocks = max(1, n_tiles * kv_heads * head_chunks)
     if blocks >= 256 or max_keys < 2 * RUN_KEYS:
         return 1
-    return max(1, min(64, 2048 // (blocks * waves), max_keys // RUN_KEYS))
+    # a step of very few rows (a single token of a model with few kv heads) takes runs of one tile of 64 keys: a run is
+    # a chain of tiles, each a round trip to memory (a decode step at batch 1 over 1,028 keys 0.896 -> 0.877 ms; at
+    # batch 8, where the chip is busier, the longer runs win, 1.337 : 1.358 ms)
+    run_keys = min(RUN_KEYS, 64) if blocks * waves <= 16 else RUN_KEYS
+    return max(1, min(64, 2048 // (blocks * waves), max_keys // run_keys))
 
 
 def bias_attention_rows() -> int:

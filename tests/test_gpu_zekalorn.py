@@ -260,7 +260,9 @@ def test_far_keys_and_edges_of_pages_and_key_runs(dtype, run_keys, monkeypatch):
     toks = random_tokens(Z.ALL[name]["vocab"], 330, 9)
     want = plain(folder, toks)
     runner = runner_for(folder, dtype)
-    assert stream.bias_attention_runs(1, 2, 1, 300, 1) == (2 if run_keys == 128 else 4)
+    # a step of very few rows cuts its keys into runs of one tile of 64 whatever RUN_KEYS says; a busier one into runs of RUN_KEYS
+    assert stream.bias_attention_runs(1, 2, 1, 300, 1) == 4
+    assert stream.bias_attention_runs(8, 2, 2, 300, 1) == (2 if run_keys == 128 else 4)
     for first in (63, 64, 65, 127, 128, 129, 7, 8, 9, 255, 257):
         rest = len(toks) - first
         steps = [{"k": first}] + [{"k": 1}] * 3 + [{"k": c} for c in cuts(rest - 3, [62, 2, 1, 64, 3])]
