@@ -65,12 +65,12 @@ BIGRAM = model(64, 97, [(scan(32, 4, 4, 2), None)], bigram=(53, 31, 7))
 
 # everything at once: a loop in the middle, both mixers, a layer without a feed-forward
 MIXED = model(96, 211, [(scan(72, 8, 6, 3), moe(16, 4, 4, shared=24)),
-                        (parallel(left(6, 2, 16, 40, 0.3, mask=(37, 5), rot=rot(16, 250000.0, (8.0, 32, 16.0, 2.0))),
+                        (parallel(left(6, 2, 16, 40, 0.3, mask=(37, 5), rot=rot(16, 300000.0, (8.0, 32, 16.0, 2.0))),
                                   right(3, 16, 32, (0.97, 0.6, 0.8)), 0.7, 1.1), moe(40, 6, 3, groups=(2, 1), shared=56)),
                         (scan(128, 32, 8, 4), None),
                         (parallel(left(5, 5, 24, 8, 0.2, mask=(9, 12), rot=rot(10, 100.0)), right(2, 20, 12, (0.5, 0.99)), 1.2, 0.4),
                          moe(32, 8, 3, groups=(4, 2)))],
-              loop=(1, 3, 2), bigram=(61, 127, 7), scale=2.0)
+              loop=(1, 3, 2), bigram=(61, 113, 5), scale=2.0)
 # the loop from the first layer to the last, three passes; a group of more heads than a workgroup's rows; keys of 32
 LOOP_ALL = model(80, 130, [(parallel(left(20, 1, 32, 32, 0.18, mask=(64, 1), rot=rot(32, 10000.0)), right(1, 64, 64, (0.9,)), 0.5, 0.5),
                             moe(32, 3, 1, shared=16)),

@@ -32,7 +32,7 @@ def draw(seed: int) -> dict:
         if r.random() < 0.8:
             dims = r.choice([d for d in (2, 4, 8, 16, 32, 64) if d <= dim] + [dim])
             scaling = (r.choice([2.0, 4.0, 16.0]), r.choice([16, 64, 512]), r.choice([4.0, 32.0]), r.choice([0.5, 1.0])) if r.random() < 0.6 else None
-            rot = Z.rot(dims, r.choice([100.0, 10000.0, 250000.0]), scaling)
+            rot = Z.rot(dims, r.choice([100.0, 10000.0, 500000.0]), scaling)
         mask = (r.choice([1, 2, 7, 16, 33, 64, 65, 100]), r.choice([0, 1, 3, 8, 70])) if r.random() < 0.85 else None
         rh = r.choice([1, 2, 3, 4])
         return Z.parallel(Z.left(heads, kv, dim, vdim, r.choice([0.1, 0.25, 0.5]), mask=mask, rot=rot),
